@@ -8,7 +8,8 @@ import importlib
 
 # architecture -> (module, class); imported lazily: some families pull in optional dependencies
 MODEL_CLASSES = {"suganex": ("localai_amd.models.suganex", "SuganexModel"),
-                 "dadizen": ("localai_amd.models.dadizen", "DadizenModel")}
+                 "dadizen": ("localai_amd.models.dadizen", "DadizenModel"),
+                 "vinozen": ("localai_amd.models.vinozen", "VinozenModel")}
 
 
 def model_class(arch: str):

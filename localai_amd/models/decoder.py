@@ -260,7 +260,9 @@ class KVCache:
         a layer without kv heads has no pages (None), one with value width 0 no V pages (its key
         rows are also its values: latent caches).  Layers with a state shape get a pool
         [state_slots, *shape] beside them, indexed by the scheduler's state slots, of the pool's
-        dtype unless the spec names one (recurrent state kept in fp32).  Slots are never cleared: a
+        dtype unless the spec names one (recurrent state kept in fp32).  A layer with several state
+        tensors gives a list of (shape, dtype or None) instead of one shape and gets a tuple of pools
+        (a convolution tail beside a recurrent state).  Slots are never cleared: a
         kernel reads of a slot only what lies at positions >= 0 of the sequence that holds it."""
         kv = cls.__new__(cls)
         kv.num_blocks, kv.block_size = num_blocks, block_size
@@ -272,8 +274,13 @@ class KVCache:
         kv.state_slots = state_slots
         kv.state = None
         if state_slots > 0:
-            kv.state = [torch.zeros(state_slots, *sp[3], dtype=sp[4] if len(sp) > 4 else dtype, device=device)
-                        if sp[3] is not None else None for sp in specs]
+            def pool(sp):
+                if sp[3] is None:
+                    return None
+                if isinstance(sp[3], list):
+                    return tuple(torch.zeros(state_slots, *shape, dtype=dt or dtype, device=device) for shape, dt in sp[3])
+                return torch.zeros(state_slots, *sp[3], dtype=sp[4] if len(sp) > 4 else dtype, device=device)
+            kv.state = [pool(sp) for sp in specs]
         return kv
 
 

@@ -120,10 +120,16 @@ def lib():
             "la_bsmoe": [I, I, P, I, I, I, P, P, I, P, I, I, I, P, P, I, LNG, I, I, P],
             "la_decode_advance": [P, P, P, P, P, P, I, I, I, P, I, P, P, P],
             "la_shortconv_kv": [I, I, P, I, P, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, P, P, P, I, I, P],
-            "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P],
-            "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P],
+            "la_attn_mix_rows": [I, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, P, I, P, P],
+            "la_attn_mix_tiles": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P, P, I, I, P, I, P, I, P, P, I, P, I, P,
+                                  P],
             "la_router_sigmoid": [I, P, LNG, P, P, I, I, I, I, I, P, P, P],
-            "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, P],
+            "la_router_topk": [I, I, P, LNG, P, P, I, I, I, I, I, P, P, P],
+            "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, I, F, F, P],
+            "la_sinusoid_add": [P, I, I, P, P, P],
+            "la_qk_norm_pages": [I, P, I, I, I, I, I, I, I, P, P, F, F, I, P, P, P, I, P],
+            "la_mamba2": [I, P, I, I, I, I, I, I, I, I, P, P, P, P, P, P, I, F, P, P, P, P, P, I, P, P, P, P, P, P, I,
+                          P],
             "la_attn_latent": [P, P, P, P, P, I, I, I, I, I, I, F, I, P, I, P, I, P, P, P],
             "la_norm_chain": [P, I, I, P, I, LNG, I, I, F, P, P, F, P, I, I, F, P, P, P, I, P],
             "la_glu_clamp": [P, I, LNG, I, I, I, F, F, P, I, P],
@@ -1845,7 +1851,8 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
              slopes: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None, chunk: int = 0,
              window: int = 0, gate: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None,
              tile_rows: int = 0, cu_q: Optional[torch.Tensor] = None, key_splits: int = 1,
-             v_width: int = 0) -> torch.Tensor:
+             v_width: int = 0, dist_bias: Optional[torch.Tensor] = None,
+             sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention with reshaped scores over paged K ([blocks, G, BS, Dk]) and V ([blocks, G, BS / 8,
     Dv, 8], transposed per 8 keys: the operand layout of the P.V matrix instruction); one
     query row per token, row r belonging to sequence row_seq[r] (block_tables row) at position
@@ -1863,9 +1870,19 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
     v_cache None with v_width > 0: a key row's first v_width columns are also its value (latent
     caches, where one stored row serves as key and value); in bf16 with one kv head, key width % 32
     and value width % 32 such calls run on the latent matrix-core kernel (key_splits as above),
-    else on the row kernel."""
+    else on the row kernel.
+    dist_bias (fp32 [N, H]): dist_bias[min(i - j, N - 1), h] is added to head h's score of key j
+    after scale and softcap (a learned bias per distance, constant from N - 1 on; see
+    bucketed_bias).  sink (fp32 [H]): the softmax denominator of head h also holds exp(sink[h]),
+    a logit without key or value that counts once per query.  Both need talk None."""
     T = q.shape[0]
     G, BS, Dk = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    if (dist_bias is not None or sink is not None) and (talk is not None or v_cache is None):
+        raise ValueError("attn_mix: distance bias and sink are not combined with the head mix or latent caches")
+    if dist_bias is not None and (dist_bias.dim() != 2 or dist_bias.shape[1] != H or dist_bias.shape[0] < 1):
+        raise ValueError("attn_mix: dist_bias is [N, H]")
+    if sink is not None and sink.numel() != H:
+        raise ValueError("attn_mix: sink is [H]")
     if v_cache is None:
         if not 0 < v_width <= Dk:
             raise ValueError("attn_mix: without V pages v_width names the value columns of a key row")
@@ -1900,7 +1917,13 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
                 s = s - slopes.float().view(H, 1) * (i - js).float().view(1, -1)
             if talk is not None:
                 s = talk.float() @ s
-            o = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+            if dist_bias is not None:
+                s = s + dist_bias.float()[(i - js).clamp(max=dist_bias.shape[0] - 1)].t()
+            if sink is not None:    # one more logit in the denominator, nothing in the numerator
+                pr = torch.softmax(torch.cat([s, sink.float().view(H, 1)], 1), -1)[:, :-1]
+            else:
+                pr = torch.softmax(s, -1)
+            o = torch.einsum("hn,nhd->hd", pr, vv)
             if gate is not None:
                 o = o * torch.sigmoid(gate[r].float()).view(H, 1)
             out[r] = o
@@ -1914,9 +1937,10 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
         raise ValueError("attn_mix: operands must be contiguous")
     for t in (row_seq, pos, block_tables):
         assert t.dtype == torch.int32 and t.is_cuda
-    for t in (slopes, talk):
-        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    for t in (slopes, talk, dist_bias, sink):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda)
     assert slopes is None or slopes.numel() == H
+    nbias = dist_bias.shape[0] if dist_bias is not None else 0
     assert talk is None or tuple(talk.shape) == (H, H)
     ldg = 0
     if gate is not None:
@@ -1954,7 +1978,7 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
                                      tiles.shape[0], cu_q.data_ptr(), pos.data_ptr(), block_tables.data_ptr(),
                                      block_tables.shape[1], H, G, Dk, Dv, BS, float(scale), float(softcap), _ptr(slopes),
                                      _ptr(talk), int(chunk), int(window), _ptr(gate), ldg, out.data_ptr(), ns,
-                                     _ptr(po), _ptr(pml), tile_rows, _stream())
+                                     _ptr(po), _ptr(pml), tile_rows, _ptr(dist_bias), nbias, _ptr(sink), _stream())
         if rc == 0:
             r0 = tile_rows
         elif rc != 1:
@@ -1966,7 +1990,8 @@ def attn_mix(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_
                                       block_tables.data_ptr(), block_tables.shape[1], T - r0, H, G, Dk, Dv, BS,
                                       float(scale), float(softcap), _ptr(slopes), _ptr(talk), int(chunk), int(window),
                                       None if gate is None else gate.data_ptr() + r0 * ldg * esz, ldg,
-                                      out.data_ptr() + r0 * H * Dv * esz, _stream()), "la_attn_mix_rows")
+                                      out.data_ptr() + r0 * H * Dv * esz, _ptr(dist_bias), nbias, _ptr(sink), _stream()),
+               "la_attn_mix_rows")
     return out
 
 
@@ -1996,11 +2021,36 @@ def router_sigmoid(xn: torch.Tensor, router: torch.Tensor, corr: Optional[torch.
     return ids, wts
 
 
+def router_softmax(xn: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], topk: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Logit router: z = xn @ router^T + bias in fp32; the topk experts with the largest z are
+    chosen (ties: lowest expert id) and weighted by the softmax over the chosen logits only.
+    Returns (ids [T, topk] int32, weights [T * topk] fp32)."""
+    T, D = xn.shape
+    E = router.shape[0]
+    if not xn.is_cuda:
+        z = xn.float() @ router.float().t()
+        if bias is not None:
+            z = z + bias.float()
+        val, idx = torch.topk(z, topk, -1)
+        return idx.to(torch.int32), torch.softmax(val, -1).reshape(-1).float()
+    assert xn.dtype in (torch.bfloat16, torch.float32) and xn.stride(1) == 1
+    assert router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == D
+    assert bias is None or (bias.dtype == torch.float32 and bias.numel() == E and bias.is_contiguous())
+    ids = torch.empty(T, topk, dtype=torch.int32, device=xn.device)
+    wts = torch.empty(T * topk, dtype=torch.float32, device=xn.device)
+    _check(lib().la_router_topk(int(xn.dtype == torch.float32), 1, xn.data_ptr(), xn.stride(0), router.data_ptr(),
+                                _ptr(bias), E, D, T, topk, 1, ids.data_ptr(), wts.data_ptr(), _stream()),
+           "la_router_topk")
+    return ids, wts
+
+
 def moe_pairs(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, ids: torch.Tensor,
-              wts: torch.Tensor) -> torch.Tensor:
+              wts: torch.Tensor, clamp: Optional[Tuple[float, float]] = None) -> torch.Tensor:
     """Routed gated experts as (token, expert) pair GEMVs on dense stacked weights (small batches,
     any width, no host sync): y[t] = sum_k wts[t, k] * Wd[e] (silu(Wg[e] x[t]) * (Wu[e] x[t])),
-    e = ids[t, k].  wg / wu [E, F, D], wd [E, D, F] in x's dtype (bf16 or fp32).  Returns fp32 [T, D]."""
+    e = ids[t, k].  wg / wu [E, F, D], wd [E, D, F] in x's dtype (bf16 or fp32).  Returns fp32 [T, D].
+    clamp = (limit, slope): the clamped unit of glu_clamp instead of SiLU gating, g = min(Wg x,
+    limit), u = clamp(Wu x, -limit, limit), g sigmoid(slope g) (u + 1)."""
     T, D = x.shape
     E, F = wg.shape[0], wg.shape[1]
     topk = ids.shape[1]
@@ -2011,8 +2061,13 @@ def moe_pairs(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Ten
         for t in range(T):
             for k in range(topk):
                 e = int(ids[t, k])
-                h = torch.nn.functional.silu(wg[e].float() @ xf[t]) * (wu[e].float() @ xf[t])
-                y[t] += wv[t, k] * (wd[e].float() @ h)
+                g_, u_ = wg[e].float() @ xf[t], wu[e].float() @ xf[t]
+                if clamp is None:
+                    h = torch.nn.functional.silu(g_) * u_
+                else:
+                    g_ = torch.clamp(g_, max=clamp[0])
+                    h = g_ * torch.sigmoid(clamp[1] * g_) * (torch.clamp(u_, -clamp[0], clamp[0]) + 1.0)
+                y[t] += wv[t, k] * (wd[e].float() @ h.to(x.dtype).float())
         return y
     for w_ in (wg, wu, wd):
         assert w_.dtype == x.dtype and w_.is_contiguous()
@@ -2021,7 +2076,9 @@ def moe_pairs(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Ten
     h = torch.empty(T * topk, F, dtype=x.dtype, device=x.device)
     y = torch.empty(T, D, dtype=torch.float32, device=x.device)
     _check(lib().la_moe_pairs(int(x.dtype == torch.float32), x.data_ptr(), wg.data_ptr(), wu.data_ptr(), wd.data_ptr(),
-                              ids.data_ptr(), wts.data_ptr(), T, topk, D, F, E, h.data_ptr(), y.data_ptr(), _stream()),
+                              ids.data_ptr(), wts.data_ptr(), T, topk, D, F, E, h.data_ptr(), y.data_ptr(),
+                              int(clamp is not None), float(clamp[0]) if clamp else 0.0, float(clamp[1]) if clamp else 0.0,
+                              _stream()),
            "la_moe_pairs")
     return y
 
@@ -2051,7 +2108,13 @@ def _branch_dense(b) -> torch.Tensor:
     return b.dense() if isinstance(b, Partial) else b.float()
 
 
-NORM_NONE, NORM_DYT, NORM_RMS, NORM_CAST = 0, 1, 2, 3
+NORM_NONE, NORM_DYT, NORM_RMS, NORM_CAST, NORM_LN = 0, 1, 2, 3, 4
+
+
+def _ln_ref(y: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = y.mean(-1, keepdim=True)
+    d = y - mu
+    return d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w.float()
 
 
 def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre: Optional[tuple] = None,
@@ -2061,11 +2124,12 @@ def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre
     place):  res <- (0 if replace else res) + post(branch) + add_vec, then returns pre(res).
     post / pre:  ("dyt", alpha, w, b): tanh(alpha x) * w + b, a norm without statistics (alpha a
     Python float, w / b fp32 [D]);  ("rms", w, eps): x / sqrt(mean(x^2) + eps) * w (post only);
-    ("cast",): res in out_dtype (pre only);  None: identity for post, no output for pre.
+    ("ln", w, eps): (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, a layer norm without bias (post
+    and pre);  ("cast",): res in out_dtype (pre only);  None: identity for post, no output for pre.
     branch: a Partial or dense [T, D] tensor (None: the stream is only read).  All arithmetic fp32."""
     T, D = res.shape
-    pm = NORM_NONE if post is None else {"dyt": NORM_DYT, "rms": NORM_RMS}[post[0]]
-    qm = NORM_NONE if pre is None else {"dyt": NORM_DYT, "cast": NORM_CAST}[pre[0]]
+    pm = NORM_NONE if post is None else {"dyt": NORM_DYT, "rms": NORM_RMS, "ln": NORM_LN}[post[0]]
+    qm = NORM_NONE if pre is None else {"dyt": NORM_DYT, "cast": NORM_CAST, "ln": NORM_LN}[pre[0]]
     if not res.is_cuda:
         if branch is not None:
             y = _branch_dense(branch)
@@ -2073,6 +2137,8 @@ def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre
                 y = torch.tanh(float(post[1]) * y) * post[2].float() + post[3].float()
             elif pm == NORM_RMS:
                 y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + float(post[2])) * post[1].float()
+            elif pm == NORM_LN:
+                y = _ln_ref(y, post[1], float(post[2]))
             if add_vec is not None:
                 y = y + add_vec.float()
             if replace:
@@ -2081,6 +2147,8 @@ def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre
                 res += y
         if qm == NORM_DYT:
             return (torch.tanh(float(pre[1]) * res) * pre[2].float() + pre[3].float()).to(out_dtype)
+        if qm == NORM_LN:
+            return _ln_ref(res, pre[1], float(pre[2])).to(out_dtype)
         return res.to(out_dtype) if qm == NORM_CAST else None
     if res.dtype != torch.float32 or not res.is_contiguous() or out_dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("norm_chain: the stream is contiguous fp32; outputs are bf16 or fp32")
@@ -2088,9 +2156,11 @@ def norm_chain(res: torch.Tensor, branch=None, post: Optional[tuple] = None, pre
     pa, pw, pb, eps = 0.0, None, None, 0.0
     if pm == NORM_DYT:
         pa, pw, pb = float(post[1]), post[2], post[3]
-    elif pm == NORM_RMS:
+    elif pm in (NORM_RMS, NORM_LN):
         pw, eps = post[1], float(post[2])
     qa, qw_, qb = (float(pre[1]), pre[2], pre[3]) if qm == NORM_DYT else (0.0, None, None)
+    if qm == NORM_LN:       # the output norm's eps travels in the slot of the squashing norm's alpha
+        qa, qw_ = float(pre[2]), pre[1]
     for t in (pw, pb, qw_, qb, add_vec):
         if t is not None and (t.dtype != torch.float32 or t.numel() != D or not t.is_contiguous()):
             raise ValueError("norm_chain: weights are contiguous fp32 [D]")
@@ -2322,6 +2392,190 @@ def retention(src: torch.Tensor, H: int, Dk: int, Dv: int, pos: torch.Tensor, cu
                               freqs.data_ptr(), float(mag), rot, float(eps), qk.data_ptr(), o.data_ptr(), out.data_ptr(),
                               _ptr(seg), max_rows, _stream()),
            "la_retention")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# Layer-list designs: additive positions, unit-normed queries and keys, bucketed distance
+# bias, state-space scan
+# ---------------------------------------------------------------------------------------
+
+def sinusoid_freqs(width: int, base: float = 10000.0, device=None) -> torch.Tensor:
+    """Angular frequencies base^(-2i / width), i = 0 .. ceil(width / 2) - 1 (float64 on the host, fp32 out)."""
+    n = (width + 1) // 2
+    return torch.from_numpy(np.power(float(base), -2.0 * np.arange(n, dtype=np.float64) / width).astype(np.float32)).to(device)
+
+
+def sinusoid_add(res: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """Additive sinusoidal positions on an fp32 stream [T, D], in place: column 2i gets
+    sin(pos * freqs[i]), column 2i + 1 cos of the same angle (angles formed and evaluated in fp32)."""
+    T, D = res.shape
+    if freqs.numel() != (D + 1) // 2 or pos.shape[0] != T or res.dtype != torch.float32:
+        raise ValueError("sinusoid_add: operand shapes do not fit")
+    if not res.is_cuda:
+        ang = pos.float()[:, None] * freqs.float()[None, :]
+        pe = torch.stack([torch.sin(ang), torch.cos(ang)], -1).reshape(T, -1)[:, :D]
+        res += pe
+        return res
+    assert res.is_contiguous() and pos.dtype == torch.int32 and freqs.dtype == torch.float32 and freqs.is_contiguous()
+    _check(lib().la_sinusoid_add(res.data_ptr(), T, D, pos.data_ptr(), freqs.data_ptr(), _stream()), "la_sinusoid_add")
+    return res
+
+
+def bucketed_bias(rel: torch.Tensor, max_dist: int) -> torch.Tensor:
+    """Distance-bias table for attn_mix from a learned bucket table rel [B, H]: row n, n = 0 ..
+    max_dist, is rel[bucket(n)] with h = B // 2 exact buckets for n < h and B - h logarithmic ones
+    up to max_dist: bucket(n) = min(B - 1, h + floor(ln(n / h) / ln(max_dist / h) * (B - h))).  From
+    max_dist on the bucket is B - 1, so attn_mix's clamp at the last row is exact.  fp32 [max_dist + 1, H]."""
+    B = rel.shape[0]
+    h = B // 2
+    idx = []
+    for n in range(int(max_dist) + 1):
+        if n < h or h == 0:
+            idx.append(min(n, B - 1))
+        elif max_dist <= h:
+            idx.append(B - 1)
+        else:
+            idx.append(min(B - 1, h + int(math.floor(math.log(n / h) / math.log(max_dist / h) * (B - h)))))
+    return rel.float()[torch.tensor(idx, dtype=torch.long, device=rel.device)].contiguous()
+
+
+def qk_norm_pages(src: torch.Tensor, H: int, Dq: int, G: int, Dk: int, Dv: int, pos: torch.Tensor,
+                  slots: Optional[torch.Tensor], eps: float, temp_coef: float = 0.0, temp_every: int = 0,
+                  k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Unit-normed queries and keys: of projection rows src [T, >= H Dq + G Dk + G Dv] (q | k | v,
+    any row stride) every query head and key head is divided by its root mean square over the head
+    (sqrt(mean x^2 + eps), no weight, fp32); queries are then multiplied by the position's
+    temperature 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) (temp_every 0: none).
+    Returns q [T, H Dq]; normed keys and the values go to the paged pools (K [blocks, G, BS, Dk],
+    V [blocks, G, BS / 8, Dv, 8]) at `slots` (-1: nowhere).  G = 0: queries only (a layer that
+    attends over another layer's pages)."""
+    T = src.shape[0]
+    Cq, Ck, Cv = H * Dq, G * Dk, G * Dv
+    if src.dim() != 2 or src.shape[1] < Cq + Ck + Cv or pos.shape[0] != T or src.stride(1) != 1:
+        raise ValueError("qk_norm_pages: operand shapes do not fit")
+    if G and (k_cache is None or v_cache is None or slots is None or tuple(k_cache.shape[1:]) != (G, k_cache.shape[2], Dk)
+              or tuple(v_cache.shape[1:]) != (G, k_cache.shape[2] // 8, Dv, 8)):
+        raise ValueError("qk_norm_pages: pools do not fit the key / value widths")
+    if not src.is_cuda:
+        x = src.float()
+        q = x[:, :Cq].reshape(T, H, Dq)
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+        if temp_every > 0:
+            tau = 1.0 + temp_coef * torch.log(torch.floor((pos.float() + 1.0) / temp_every) + 1.0)
+            q = q * tau.view(T, 1, 1)
+        if G:
+            k = x[:, Cq:Cq + Ck].reshape(T, G, Dk)
+            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+            _page_write_ref(k_cache, v_cache, slots, k, x[:, Cq + Ck:Cq + Ck + Cv].reshape(T, G, Dv))
+        return q.reshape(T, Cq).to(src.dtype)
+    f32 = src.dtype == torch.float32
+    if src.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("qk_norm_pages: bf16 or fp32 rows")
+    if G and (k_cache.dtype != src.dtype or v_cache.dtype != src.dtype):
+        raise ValueError("qk_norm_pages: pools share the rows' dtype")
+    assert pos.dtype == torch.int32 and (slots is None or (slots.dtype == torch.int32 and slots.shape[0] == T))
+    q = torch.empty(T, Cq, dtype=src.dtype, device=src.device)
+    _check(lib().la_qk_norm_pages(int(f32), src.data_ptr(), src.stride(0), T, H, Dq, G, Dk, Dv, pos.data_ptr(), _ptr(slots),
+                                  float(eps), float(temp_coef), int(temp_every), q.data_ptr(), _ptr(k_cache), _ptr(v_cache),
+                                  k_cache.shape[2] if G else 0, _stream()), "la_qk_norm_pages")
+    return q
+
+
+def mamba2_states(slots: int, H: int, P: int, N: int, G: int, taps: int, dtype=torch.bfloat16, device=None):
+    """State pools of ops.mamba2: (convolution tails [slots, taps - 1, H P + 2 G N] of the activation
+    dtype, recurrent state fp32 [slots, H, P, N], a head's N x P state stored value-column major)."""
+    return (torch.zeros(slots, max(taps - 1, 0), H * P + 2 * G * N, dtype=dtype, device=device),
+            torch.zeros(slots, H, P, N, dtype=torch.float32, device=device))
+
+
+def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tensor, conv_b: Optional[torch.Tensor],
+           dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, norm_w: torch.Tensor, norm_groups: int,
+           eps: float, pos: torch.Tensor, cu_q: torch.Tensor, sslots: torch.Tensor, conv_state: torch.Tensor,
+           ssm_state: torch.Tensor, max_rows: int = 0) -> torch.Tensor:
+    """State-space mixer with a scalar decay per head (state-space duality form) over projection
+    rows src [T, 2 H P + 2 G N + H] laid out [z | x | B | C | dt]:
+      * x, B, C pass a depthwise causal convolution over time (conv_w [H P + 2 G N, taps] fp32, last
+        tap = current token, bias conv_b, zeros before position 0) and silu;
+      * dt = softplus(dt + dt_bias) (no clamp); per head h (group floor(h / (H / G))):
+        S <- exp(-exp(a_log[h]) dt) S + dt B x^T (N x P),  y = S^T C + d_skip[h] x;
+      * y times silu(z), then divided by the root mean square of each of `norm_groups` equal parts
+        of the H P channels (eps), times norm_w.
+    Rows of a sequence portion are consecutive (cu_q [nseq + 1], pos [T]); the portion's history
+    comes from conv_state[sslots[seq]] (the last taps - 1 rows of [x | B | C] before the
+    convolution) and ssm_state[sslots[seq]] (fp32), both taken as zero before position 0, and both
+    are advanced to the portion's end.  dt, decays, the recurrence, its state and outputs, the gate
+    and the norm are fp32.  Returns [T, H P] in src's dtype."""
+    T = src.shape[0]
+    nseq = cu_q.shape[0] - 1
+    inner, GN = H * P, G * N
+    C = inner + 2 * GN
+    taps = conv_w.shape[1]
+    if (src.dim() != 2 or src.shape[1] != 2 * inner + 2 * GN + H or H % G or inner % norm_groups or conv_w.shape[0] != C
+            or tuple(conv_state.shape[1:]) != (max(taps - 1, 0), C) or tuple(ssm_state.shape[1:]) != (H, P, N)
+            or dt_bias.numel() != H or a_log.numel() != H or d_skip.numel() != H or norm_w.numel() != inner
+            or sslots.shape[0] != nseq or pos.shape[0] != T or (conv_b is not None and conv_b.numel() != C)):
+        raise ValueError("mamba2: operand shapes do not fit")
+    if not src.is_cuda:
+        u = src.float()
+        z, xbc, dt = u[:, :inner], u[:, inner:inner + C], u[:, inner + C:]
+        dt = torch.nn.functional.softplus(dt + dt_bias.float(), threshold=1e9)
+        dec = torch.exp(-torch.exp(a_log.float()) * dt)                       # [T, H]
+        y = torch.zeros(T, H, P)
+        cu = cu_q.tolist()
+        rep = H // G
+        for s in range(nseq):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            ss, p0 = int(sslots[s]), int(pos[a])
+            hist = torch.zeros(taps - 1, C)
+            if taps > 1:
+                hist = conv_state[ss].float().clone()
+                for i in range(taps - 1):            # state row i holds position p0 - (taps - 1) + i
+                    if p0 - (taps - 1) + i < 0:
+                        hist[i] = 0
+            ext = torch.cat([hist, xbc[a:b]], 0)
+            c = torch.zeros(b - a, C) if conv_b is None else conv_b.float().repeat(b - a, 1)
+            for j in range(taps):
+                c = c + conv_w[:, j].float() * ext[j:j + (b - a)]
+            c = torch.nn.functional.silu(c)
+            if taps > 1:
+                conv_state[ss] = ext[-(taps - 1):].to(conv_state.dtype)
+            xs = c[:, :inner].reshape(-1, H, P)
+            Bm = c[:, inner:inner + GN].reshape(-1, G, N).repeat_interleave(rep, 1)
+            Cm = c[:, inner + GN:].reshape(-1, G, N).repeat_interleave(rep, 1)
+            S = torch.zeros(H, P, N) if p0 == 0 else ssm_state[ss].float().clone()
+            for t in range(b - a):
+                S = dec[a + t].view(H, 1, 1) * S + (dt[a + t].view(H, 1) * xs[t]).unsqueeze(2) * Bm[t].unsqueeze(1)
+                y[a + t] = torch.einsum("hpn,hn->hp", S, Cm[t]) + d_skip.float().view(H, 1) * xs[t]
+            ssm_state[ss] = S
+        yg = (y.reshape(T, inner) * torch.nn.functional.silu(z)).reshape(T, norm_groups, inner // norm_groups)
+        yg = yg * torch.rsqrt(yg.pow(2).mean(-1, keepdim=True) + eps)
+        return (yg.reshape(T, inner) * norm_w.float()).to(src.dtype)
+    f32 = src.dtype == torch.float32
+    if src.dtype not in (torch.float32, torch.bfloat16) or not src.is_contiguous() or conv_state.dtype != src.dtype:
+        raise ValueError("mamba2: contiguous bf16 or fp32 rows, convolution tails of the same dtype")
+    if ssm_state.dtype != torch.float32 or not ssm_state.is_contiguous() or not conv_state.is_contiguous():
+        raise ValueError("mamba2: the recurrent state pool is contiguous fp32")
+    for t in (pos, cu_q, sslots):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    for t in (conv_w, conv_b, dt_bias, a_log, d_skip, norm_w):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda)
+    dev = src.device
+    xs = torch.empty(T, inner, dtype=torch.float32, device=dev)         # convolved x
+    cb = torch.empty(T, 2 * GN, dtype=torch.float32, device=dev)        # convolved C | B: the scan's q | k rows
+    dtd = torch.empty(T, 2 * H, dtype=torch.float32, device=dev)        # dt | decay per (token, head)
+    o = torch.empty(T, inner, dtype=torch.float32, device=dev)
+    out = torch.empty(T, inner, dtype=src.dtype, device=dev)
+    max_rows = int(max_rows) if max_rows > 0 else T
+    seg = torch.empty((T // RETENTION_SEG + nseq) * H * P * N, dtype=torch.float32, device=dev) \
+        if (T >= 8 * RETENTION_SEG and max_rows >= 4 * RETENTION_SEG) else None
+    _check(lib().la_mamba2(int(f32), src.data_ptr(), T, nseq, H, P, N, G, taps, ssm_state.shape[0], conv_w.data_ptr(),
+                           _ptr(conv_b), dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), norm_w.data_ptr(),
+                           int(norm_groups), float(eps), pos.data_ptr(), cu_q.data_ptr(), sslots.data_ptr(),
+                           conv_state.data_ptr(), ssm_state.data_ptr(), int(T == nseq), xs.data_ptr(), cb.data_ptr(),
+                           dtd.data_ptr(), o.data_ptr(), out.data_ptr(), _ptr(seg), max_rows, _stream()), "la_mamba2")
     return out
 
 

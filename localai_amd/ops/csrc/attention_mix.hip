@@ -57,7 +57,8 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
     const AT* __restrict__ q, const AT* __restrict__ kc, const AT* __restrict__ vc, const int* __restrict__ row_seq,
     const int* __restrict__ pos, const int* __restrict__ bt, int maxb, int H, int G, int Dk, int Dv, int BS,
     float scale, float softcap, const float* __restrict__ slopes, const float* __restrict__ talk, int chunk,
-    int window, const AT* __restrict__ gate, int ldg, AT* __restrict__ out) {
+    int window, const AT* __restrict__ gate, int ldg, AT* __restrict__ out, const float* __restrict__ dbias, int nbias,
+    const float* __restrict__ sink) {
   extern __shared__ float lds[];
   float* qs = lds;                       // [H][Dk]
   float* s1 = qs + H * Dk;               // [H][KT] raw scores
@@ -71,7 +72,8 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
   const int rep = H / G;
   const bool vec = (Dk * sizeof(AT)) % 16 == 0;
   for (int e = tid; e < H * Dk; e += AM_NT) qs[e] = (float)q[(long)r * H * Dk + e];
-  for (int h = tid; h < H; h += AM_NT) { mrun[h] = -INFINITY; lrun[h] = 0.f; }
+  // a sink is a logit without key or value: the running (max, sum) start at (sink, 1) instead of (-inf, 0)
+  for (int h = tid; h < H; h += AM_NT) { mrun[h] = sink ? sink[h] : -INFINITY; lrun[h] = sink ? 1.f : 0.f; }
   int lo = 0;
   if (chunk > 0) lo = (i / chunk) * chunk;
   if (window > 0) lo = max(lo, i - window + 1);
@@ -91,6 +93,7 @@ __global__ __launch_bounds__(AM_NT) void attn_mix_rows_kernel(
         s = dot_row<AT>(qs + h * Dk, kc + (((long)blk * G + g) * BS + off) * Dk, Dk, vec) * scale;
         if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         if (slopes) s -= slopes[h] * (float)(i - j);
+        if (dbias) s += dbias[(long)min(i - j, nbias - 1) * H + h];
       }
       s1[e] = s;
     }
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
     const int* __restrict__ bt, int maxb, int H, int G, int Dk, int Dv, int BS, float scale, float softcap,
     const float* __restrict__ slopes, const float* __restrict__ talk, int chunk, int window,
     const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out, int nsplit, float* __restrict__ part_o,
-    float* __restrict__ part_ml) {
+    float* __restrict__ part_ml, const float* __restrict__ dbias, int nbias, const float* __restrict__ sink) {
   extern __shared__ float lds[];
   float* s1 = lds;                           // [H][16][AT_SS]
   float* mrun = s1 + H * 16 * AT_SS;         // [H * 16]
@@ -203,7 +206,9 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
   const int* tab = bt + (long)seq * maxb;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fr = lane & 15, fq = lane >> 4;
   const int rep = H / G, KC = Dk / 32;
-  for (int e = tid; e < H * 16; e += NW * 64) { mrun[e] = -INFINITY; lrun[e] = 0.f; }
+  // sink: a logit without key or value, counted once per (head, query) -- by the first key split
+  const bool sunk = sink != nullptr && blockIdx.y == 0;
+  for (int e = tid; e < H * 16; e += NW * 64) { mrun[e] = sunk ? sink[e >> 4] : -INFINITY; lrun[e] = sunk ? 1.f : 0.f; }
   f32x4 o[HPW][NDV];
 #pragma unroll
   for (int a = 0; a < HPW; ++a)
@@ -291,6 +296,7 @@ __global__ __launch_bounds__(NW * 64) void attn_mix_tile_kernel(
             float sc = a[i] * scale;
             if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
             sc -= slope * (float)(qpos - key);
+            if (dbias) sc += dbias[(long)min(max(qpos - key, 0), nbias - 1) * H + h];
             if (key > qpos || qr >= nrow) sc = 0.f;   // hidden below; finite for the mix
             *sp = sc;
           }
@@ -500,13 +506,14 @@ template <int NW, int HPW, int NDV>
 static int launch_tile(int nsplit, void* part_o, void* part_ml, int ntiles, size_t shm, hipStream_t s, const void* q, const void* kc, const void* vc,
                        const void* tiles, const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G,
                        int Dk, int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
-                       int chunk, int window, const void* gate, int ldg, void* out) {
+                       int chunk, int window, const void* gate, int ldg, void* out, const void* dbias, int nbias,
+                       const void* sink) {
   auto k = attn_mix_tile_kernel<NW, HPW, NDV>;
   if (shm > 48 * 1024) (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
   hipLaunchKernelGGL(k, dim3(ntiles, nsplit), dim3(NW * 64), shm, s, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,
                      (const int*)tiles, (const int*)cu_q, (const int*)pos, (const int*)bt, maxb, H, G, Dk, Dv, BS, scale,
                      softcap, (const float*)slopes, (const float*)talk, chunk, window, (const bf16*)gate, ldg,
-                     (bf16*)out, nsplit, (float*)part_o, (float*)part_ml);
+                     (bf16*)out, nsplit, (float*)part_o, (float*)part_ml, (const float*)dbias, nbias, (const float*)sink);
   return (int)hipGetLastError();
 }
 
@@ -515,9 +522,10 @@ static int launch_tile(int nsplit, void* part_o, void* part_ml, int ntiles, size
 extern "C" int la_attn_mix_rows(int f32, const void* q, const void* kc, const void* vc, const void* row_seq,
                                 const void* pos, const void* bt, int maxb, int T, int H, int G, int Dk, int Dv, int BS,
                                 float scale, float softcap, const void* slopes, const void* talk, int chunk, int window,
-                                const void* gate, int ldg, void* out, void* stream) {
+                                const void* gate, int ldg, void* out, const void* dbias, int nbias, const void* sink,
+                                void* stream) {
   using namespace la;
-  if (T <= 0 || H <= 0 || G <= 0 || H % G || H * Dv > AM_NT * AM_MAXO) return -1;
+  if (T <= 0 || H <= 0 || G <= 0 || H % G || H * Dv > AM_NT * AM_MAXO || (dbias && nbias < 1)) return -1;
   const size_t shm = sizeof(float) * ((size_t)H * Dk + 2 * (size_t)H * AM_KT + 3 * (size_t)H);
   if (shm > 160 * 1024) return -2;
   hipStream_t s = (hipStream_t)stream;
@@ -527,14 +535,14 @@ extern "C" int la_attn_mix_rows(int f32, const void* q, const void* kc, const vo
     hipLaunchKernelGGL((attn_mix_rows_kernel<float>), dim3(T), dim3(AM_NT), shm, s, (const float*)q, (const float*)kc,
                        (const float*)vc, (const int*)row_seq, (const int*)pos, (const int*)bt, maxb, H, G, Dk, Dv, BS,
                        scale, softcap, (const float*)slopes, (const float*)talk, chunk, window, (const float*)gate, ldg,
-                       (float*)out);
+                       (float*)out, (const float*)dbias, nbias, (const float*)sink);
   } else {
     if (shm > 48 * 1024)
       (void)hipFuncSetAttribute((const void*)attn_mix_rows_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
     hipLaunchKernelGGL((attn_mix_rows_kernel<bf16>), dim3(T), dim3(AM_NT), shm, s, (const bf16*)q, (const bf16*)kc,
                        (const bf16*)vc, (const int*)row_seq, (const int*)pos, (const int*)bt, maxb, H, G, Dk, Dv, BS,
                        scale, softcap, (const float*)slopes, (const float*)talk, chunk, window, (const bf16*)gate, ldg,
-                       (bf16*)out);
+                       (bf16*)out, (const float*)dbias, nbias, (const float*)sink);
   }
   return (int)hipGetLastError();
 }
@@ -549,9 +557,10 @@ extern "C" int la_attn_mix_tiles(const void* q, const void* kc, const void* vc, 
                                  const void* cu_q, const void* pos, const void* bt, int maxb, int H, int G, int Dk,
                                  int Dv, int BS, float scale, float softcap, const void* slopes, const void* talk,
                                  int chunk, int window, const void* gate, int ldg, void* out, int nsplit, void* part_o,
-                                 void* part_ml, int rows, void* stream) {
+                                 void* part_ml, int rows, const void* dbias, int nbias, const void* sink, void* stream) {
   using namespace la;
-  if (ntiles <= 0 || H <= 0 || G <= 0 || H % G || nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml)))
+  if (ntiles <= 0 || H <= 0 || G <= 0 || H % G || nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_o || !part_ml)) ||
+      (dbias && nbias < 1))
     return -1;
   if ((Dk % 32) || (Dv % 16) || Dv > 128 || H > 32 || (BS & 7)) return 1;
   const size_t shm = (size_t)H * 16 * (AT_SS * 4 + 3 * 4 + AT_PS * 2);
@@ -563,7 +572,8 @@ extern "C" int la_attn_mix_tiles(const void* q, const void* kc, const void* vc, 
 #define LA_TILE(NW, HPW, NDV)                                                                                      \
   if (rc == 1 && nw == NW && hpw <= HPW && ndv == NDV)                                                             \
     rc = launch_tile<NW, HPW, NDV>(nsplit, part_o, part_ml, ntiles, shm, s, q, kc, vc, tiles, cu_q, pos, bt, maxb, H, \
-                                   G, Dk, Dv, BS, scale, softcap, slopes, talk, chunk, window, gate, ldg, out);
+                                   G, Dk, Dv, BS, scale, softcap, slopes, talk, chunk, window, gate, ldg, out, dbias,    \
+                                   nbias, sink);
   LA_TILE(4, 1, 2) LA_TILE(4, 1, 4) LA_TILE(4, 1, 8) LA_TILE(4, 2, 2) LA_TILE(4, 2, 4) LA_TILE(4, 2, 8)
   LA_TILE(8, 2, 2) LA_TILE(8, 2, 4) LA_TILE(8, 2, 8) LA_TILE(8, 4, 2) LA_TILE(8, 4, 4) LA_TILE(8, 4, 8)
 #undef LA_TILE

@@ -1,5 +1,6 @@
 // Mixture-of-experts pieces for dense (bf16 / fp32) expert weights of any width:
-//   * a router with sigmoid scores, an optional selection-only correction and normalised weights;
+//   * a router with sigmoid scores, an optional selection-only correction and normalised weights,
+//     or with biased logits and the softmax over the chosen logits as weights;
 //   * the routed experts of small batches as (token, expert) pair GEMVs: gate|up with the SiLU
 //     gating fused, then the down projection with the weighted top-k combine fused, no atomics.
 // Larger batches group rows by expert and run library GEMMs (the caller's choice).
@@ -7,14 +8,17 @@
 
 namespace la {
 
-// One wave per token: z_e = router[e] . x (fp32), s = sigmoid(z); the `topk` largest s + corr are
-// chosen (ties: lowest expert id), their weights are s / (sum of the chosen s + 1e-20).
+// One wave per token: z_e = router[e] . x (fp32).
+// mode 0: s = sigmoid(z); the `topk` largest s + corr are chosen (ties: lowest expert id), their
+//         weights are s / (sum of the chosen s + 1e-20).
+// mode 1: s = z + corr (a bias that counts in the weights too); the `topk` largest s are chosen,
+//         their weights are the softmax over the chosen s.
 template <typename AT>
-__global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restrict__ x, long ldx,
-                                                             const float* __restrict__ router,
-                                                             const float* __restrict__ corr, int E, int D, int T,
-                                                             int topk, int renorm, int* __restrict__ ids,
-                                                             float* __restrict__ wts) {
+__global__ __launch_bounds__(256) void router_topk_kernel(const AT* __restrict__ x, long ldx,
+                                                          const float* __restrict__ router,
+                                                          const float* __restrict__ corr, int E, int D, int T,
+                                                          int topk, int renorm, int mode, int* __restrict__ ids,
+                                                          float* __restrict__ wts) {
   __shared__ float sc[4][256];
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + w;
@@ -47,11 +51,11 @@ __global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restric
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const float v = wave_sum(a[k]);
-      if (lane == 0 && e0 + k < E) sc[w][e0 + k] = 1.f / (1.f + __expf(-v));
+      if (lane == 0 && e0 + k < E) sc[w][e0 + k] = mode ? v + (corr ? corr[e0 + k] : 0.f) : 1.f / (1.f + __expf(-v));
     }
   }
   __syncthreads();
-  float sum = 0.f, my_s = 0.f;
+  float sum = 0.f, my_s = 0.f, top0 = 0.f;
   int my_id = 0;
   uint32_t taken = 0;   // bit i: this lane's expert e = lane + 64 * i is already chosen
   for (int k = 0; k < topk; ++k) {
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restric
     for (int i = 0; i < 4; ++i) {
       const int e = lane + 64 * i;
       if (e < E && !((taken >> i) & 1u)) {
-        const float c = sc[w][e] + (corr ? corr[e] : 0.f);
+        const float c = sc[w][e] + ((corr && !mode) ? corr[e] : 0.f);
         if (c > best || (c == best && e < bi)) { best = c; bi = e; }
       }
     }
@@ -70,21 +74,27 @@ __global__ __launch_bounds__(256) void router_sigmoid_kernel(const AT* __restric
       if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
     }
     if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
-    const float s = sc[w][bi];
+    float s = sc[w][bi];
+    if (mode) {           // softmax over the chosen logits: the first chosen one is the largest
+      if (k == 0) top0 = s;
+      s = expf(s - top0);
+    }
     sum += s;
     if (lane == k) { my_s = s; my_id = bi; }
   }
   if (live && lane < topk) {
     ids[(long)t * topk + lane] = my_id;
-    wts[(long)t * topk + lane] = renorm ? my_s / (sum + 1e-20f) : my_s;
+    wts[(long)t * topk + lane] = (renorm || mode) ? my_s / (sum + 1e-20f) : my_s;
   }
 }
 
-// h[p][f] = silu(Wg[e_p][f] . x[t_p]) * (Wu[e_p][f] . x[t_p]),  p = t * topk + slot; a wave per (p, f)
+// h[p][f] = silu(Wg[e_p][f] . x[t_p]) * (Wu[e_p][f] . x[t_p]),  p = t * topk + slot; a wave per (p, f).
+// clamp: g = min(Wg x, limit), u = clamp(Wu x, -limit, limit), h = g sigmoid(slope g) (u + 1) instead.
 template <typename AT, typename WT>
 __global__ __launch_bounds__(256) void moe_pair_glu_kernel(const AT* __restrict__ x, const WT* __restrict__ wg,
                                                            const WT* __restrict__ wu, const int* __restrict__ ids,
-                                                           int topk, int D, int F, int E, AT* __restrict__ h) {
+                                                           int topk, int D, int F, int E, AT* __restrict__ h, int clamp,
+                                                           float limit, float slope) {
   const int p = blockIdx.y;
   const int f = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (f >= F) return;
@@ -101,7 +111,16 @@ __global__ __launch_bounds__(256) void moe_pair_glu_kernel(const AT* __restrict_
   }
   a = wave_sum(a);
   b = wave_sum(b);
-  if (lane == 0) h[(long)p * F + f] = (AT)(silu(a) * b);
+  if (lane == 0) {
+    float v;
+    if (clamp) {
+      const float g2 = fminf(a, limit), u2 = fminf(fmaxf(b, -limit), limit);
+      v = g2 / (1.f + expf(-slope * g2)) * (u2 + 1.f);
+    } else {
+      v = silu(a) * b;
+    }
+    h[(long)p * F + f] = (AT)v;
+  }
 }
 
 // y[t][d] = sum_slot w[p] * (Wd[e_p][d] . h[p]); a wave per (t, d), slots in order (deterministic)
@@ -127,24 +146,30 @@ __global__ __launch_bounds__(256) void moe_pair_down_kernel(const AT* __restrict
 
 }  // namespace la
 
-extern "C" int la_router_sigmoid(int f32, const void* x, long ldx, const void* router, const void* corr, int E, int D,
-                                 int T, int topk, int renorm, void* ids, void* wts, void* stream) {
+extern "C" int la_router_topk(int f32, int mode, const void* x, long ldx, const void* router, const void* corr, int E,
+                              int D, int T, int topk, int renorm, void* ids, void* wts, void* stream) {
   using namespace la;
-  if (E < 1 || E > 256 || topk < 1 || topk > E || topk > 64 || T <= 0) return -1;
+  if (E < 1 || E > 256 || topk < 1 || topk > E || topk > 64 || T <= 0 || mode < 0 || mode > 1) return -1;
   dim3 grid((T + 3) / 4);
   if (f32)
-    hipLaunchKernelGGL((router_sigmoid_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, ldx,
-                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, (int*)ids, (float*)wts);
+    hipLaunchKernelGGL((router_topk_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, ldx,
+                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, mode, (int*)ids, (float*)wts);
   else
-    hipLaunchKernelGGL((router_sigmoid_kernel<bf16>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, ldx,
-                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, (int*)ids, (float*)wts);
+    hipLaunchKernelGGL((router_topk_kernel<bf16>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, ldx,
+                       (const float*)router, (const float*)corr, E, D, T, topk, renorm, mode, (int*)ids, (float*)wts);
   return (int)hipGetLastError();
+}
+
+extern "C" int la_router_sigmoid(int f32, const void* x, long ldx, const void* router, const void* corr, int E, int D,
+                                 int T, int topk, int renorm, void* ids, void* wts, void* stream) {
+  return la_router_topk(f32, 0, x, ldx, router, corr, E, D, T, topk, renorm, ids, wts, stream);
 }
 
 // f32: activations and weights fp32 (else both bf16).  x [T, D], wg / wu [E, F, D], wd [E, D, F],
 // ids [T * topk], wts [T * topk] -> h [T * topk, F] (scratch, activation type), y [T, D] fp32.
 extern "C" int la_moe_pairs(int f32, const void* x, const void* wg, const void* wu, const void* wd, const void* ids,
-                            const void* wts, int T, int topk, int D, int F, int E, void* h, void* y, void* stream) {
+                            const void* wts, int T, int topk, int D, int F, int E, void* h, void* y, int clamp, float limit,
+                            float slope, void* stream) {
   using namespace la;
   if (T <= 0 || topk < 1 || D < 1 || F < 1) return -1;
   const int P = T * topk;
@@ -153,12 +178,12 @@ extern "C" int la_moe_pairs(int f32, const void* x, const void* wg, const void* 
   hipStream_t s = (hipStream_t)stream;
   if (f32) {
     hipLaunchKernelGGL((moe_pair_glu_kernel<float, float>), g1, dim3(256), 0, s, (const float*)x, (const float*)wg,
-                       (const float*)wu, (const int*)ids, topk, D, F, E, (float*)h);
+                       (const float*)wu, (const int*)ids, topk, D, F, E, (float*)h, clamp, limit, slope);
     hipLaunchKernelGGL((moe_pair_down_kernel<float, float>), g2, dim3(256), 0, s, (const float*)h, (const float*)wd,
                        (const int*)ids, (const float*)wts, topk, D, F, E, (float*)y);
   } else {
     hipLaunchKernelGGL((moe_pair_glu_kernel<bf16, bf16>), g1, dim3(256), 0, s, (const bf16*)x, (const bf16*)wg,
-                       (const bf16*)wu, (const int*)ids, topk, D, F, E, (bf16*)h);
+                       (const bf16*)wu, (const int*)ids, topk, D, F, E, (bf16*)h, clamp, limit, slope);
     hipLaunchKernelGGL((moe_pair_down_kernel<bf16, bf16>), g2, dim3(256), 0, s, (const bf16*)h, (const bf16*)wd,
                        (const int*)ids, (const float*)wts, topk, D, F, E, (float*)y);
   }

@@ -3,7 +3,8 @@
 //
 //   norm_chain:  res <- (replace ? 0 : res) + post(branch) + add_vec;  out = pre(res)
 //       post:  none | dyt: tanh(alpha y) * w + b | rms: y / sqrt(mean(y^2) + eps) * w
-//       pre:   none | dyt | cast (the stream itself in the output type)
+//              | ln: (y - mean) / sqrt(mean((y - mean)^2) + eps) * w  (layer norm, no bias)
+//       pre:   none | dyt | cast (the stream itself in the output type) | ln (eps in the alpha slot)
 //     one launch where a pre-normed stream has "add + norm": the branch's own norm, the residual
 //     add and the next sublayer's input norm.  A workgroup per row; the rms variant reads the
 //     branch row twice (second time from cache) instead of holding it in registers, so any width runs.
@@ -38,7 +39,7 @@ LA_DEV void put(void* out, int out_f32, long idx, float v) {
   else ((bf16*)out)[idx] = (bf16)v;
 }
 
-enum { NC_NONE = 0, NC_DYT = 1, NC_RMS = 2, NC_CAST = 3 };
+enum { NC_NONE = 0, NC_DYT = 1, NC_RMS = 2, NC_CAST = 3, NC_LN = 4 };
 constexpr int NC_NT = 256;
 
 __global__ __launch_bounds__(NC_NT) void norm_chain_kernel(float* __restrict__ res, int D, RowSrc src, int has_src,
@@ -51,11 +52,16 @@ __global__ __launch_bounds__(NC_NT) void norm_chain_kernel(float* __restrict__ r
   __shared__ float red[NC_NT / 64];
   const int t = blockIdx.x, tid = threadIdx.x;
   const long base = (long)t * D;
-  float inv = 1.f;
-  if (has_src && post == NC_RMS) {
+  float inv = 1.f, mean = 0.f;
+  if (has_src && (post == NC_RMS || post == NC_LN)) {
+    if (post == NC_LN) {
+      float sm = 0.f;
+      for (int c = tid; c < D; c += NC_NT) sm += src_at(src, base + c);
+      mean = block_sum<NC_NT>(sm, red) / (float)D;
+    }
     float ss = 0.f;
     for (int c = tid; c < D; c += NC_NT) {
-      const float y = src_at(src, base + c);
+      const float y = src_at(src, base + c) - mean;
       ss = fmaf(y, y, ss);
     }
     ss = block_sum<NC_NT>(ss, red);
@@ -66,13 +72,25 @@ __global__ __launch_bounds__(NC_NT) void norm_chain_kernel(float* __restrict__ r
     if (has_src) {
       float y = src_at(src, base + c);
       if (post == NC_DYT) y = fmaf(tanhf(pa * y), pw[c], pb[c]);
-      else if (post == NC_RMS) y = y * inv * pw[c];
+      else if (post == NC_RMS || post == NC_LN) y = (y - mean) * inv * pw[c];
       if (addv) y += addv[c];
       x = replace ? y : x + y;
       res[base + c] = x;
     }
     if (pre == NC_DYT) put(out, out_f32, base + c, fmaf(tanhf(qa * x), qw[c], qb[c]));
     else if (pre == NC_CAST) put(out, out_f32, base + c, x);
+  }
+  if (pre == NC_LN) {   // layer norm of the updated row: every thread re-reads the columns it wrote
+    float sm = 0.f;
+    for (int c = tid; c < D; c += NC_NT) sm += res[base + c];
+    const float m2 = block_sum<NC_NT>(sm, red) / (float)D;
+    float ss = 0.f;
+    for (int c = tid; c < D; c += NC_NT) {
+      const float d = res[base + c] - m2;
+      ss = fmaf(d, d, ss);
+    }
+    const float inv2 = 1.f / sqrtf(block_sum<NC_NT>(ss, red) / (float)D + qa);
+    for (int c = tid; c < D; c += NC_NT) put(out, out_f32, base + c, (res[base + c] - m2) * inv2 * qw[c]);
   }
 }
 
@@ -97,14 +115,23 @@ __global__ __launch_bounds__(NC_NT) void norm_chain4_kernel(float* __restrict__ 
       for (int j = 0; j < 4; ++j) y[j] = (float)v[j];
     }
   };
-  float inv = 1.f;
-  if (has_src && post == NC_RMS) {
+  float inv = 1.f, mean = 0.f;
+  if (has_src && (post == NC_RMS || post == NC_LN)) {
+    if (post == NC_LN) {
+      float sm = 0.f;
+      for (int c = tid * 4; c < D; c += NC_NT * 4) {
+        float y[4];
+        load(c, y);
+        sm += (y[0] + y[1]) + (y[2] + y[3]);
+      }
+      mean = block_sum<NC_NT>(sm, red) / (float)D;
+    }
     float ss = 0.f;
     for (int c = tid * 4; c < D; c += NC_NT * 4) {
       float y[4];
       load(c, y);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) ss = fmaf(y[j], y[j], ss);
+      for (int j = 0; j < 4; ++j) ss = fmaf(y[j] - mean, y[j] - mean, ss);
     }
     ss = block_sum<NC_NT>(ss, red);
     inv = 1.f / sqrtf(ss / (float)D + eps);
@@ -118,16 +145,40 @@ __global__ __launch_bounds__(NC_NT) void norm_chain4_kernel(float* __restrict__ 
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (post == NC_DYT) y[j] = fmaf(tanhf(pa * y[j]), pw[c + j], pb[c + j]);
-        else if (post == NC_RMS) y[j] = y[j] * inv * pw[c + j];
+        else if (post == NC_RMS || post == NC_LN) y[j] = (y[j] - mean) * inv * pw[c + j];
         if (addv) y[j] += addv[c + j];
         x[j] = replace ? y[j] : x[j] + y[j];
       }
       *(float4*)(res + base + c) = make_float4(x[0], x[1], x[2], x[3]);
     }
-    if (pre != NC_NONE) {
+    if (pre == NC_DYT || pre == NC_CAST) {
       float o[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) o[j] = pre == NC_DYT ? fmaf(tanhf(qa * x[j]), qw[c + j], qb[c + j]) : x[j];
+      if (out_f32) *(float4*)((float*)out + base + c) = make_float4(o[0], o[1], o[2], o[3]);
+      else {
+        bf16x4 ob = {(bf16)o[0], (bf16)o[1], (bf16)o[2], (bf16)o[3]};
+        *(bf16x4*)((bf16*)out + base + c) = ob;
+      }
+    }
+  }
+  if (pre == NC_LN) {   // layer norm of the updated row: every thread re-reads the columns it wrote
+    float sm = 0.f;
+    for (int c = tid * 4; c < D; c += NC_NT * 4) {
+      const float4 v = *(const float4*)(res + base + c);
+      sm += (v.x + v.y) + (v.z + v.w);
+    }
+    const float m2 = block_sum<NC_NT>(sm, red) / (float)D;
+    float ss = 0.f;
+    for (int c = tid * 4; c < D; c += NC_NT * 4) {
+      const float4 v = *(const float4*)(res + base + c);
+      ss = fmaf(v.x - m2, v.x - m2, fmaf(v.y - m2, v.y - m2, fmaf(v.z - m2, v.z - m2, fmaf(v.w - m2, v.w - m2, ss))));
+    }
+    const float inv2 = 1.f / sqrtf(block_sum<NC_NT>(ss, red) / (float)D + qa);
+    for (int c = tid * 4; c < D; c += NC_NT * 4) {
+      const float4 v = *(const float4*)(res + base + c);
+      const float o[4] = {(v.x - m2) * inv2 * qw[c], (v.y - m2) * inv2 * qw[c + 1], (v.z - m2) * inv2 * qw[c + 2],
+                          (v.w - m2) * inv2 * qw[c + 3]};
       if (out_f32) *(float4*)((float*)out + base + c) = make_float4(o[0], o[1], o[2], o[3]);
       else {
         bf16x4 ob = {(bf16)o[0], (bf16)o[1], (bf16)o[2], (bf16)o[3]};
@@ -187,8 +238,9 @@ extern "C" int la_norm_chain(void* res, int T, int D, const void* sp, int src_f3
   using namespace la;
   if (T <= 0 || D <= 0 || !res) return -1;
   if (post == NC_DYT && (!pw || !pb)) return -2;
-  if (post == NC_RMS && !pw) return -2;
+  if ((post == NC_RMS || post == NC_LN) && !pw) return -2;
   if (pre == NC_DYT && (!qw || !qb)) return -2;
+  if (pre == NC_LN && !qw) return -2;
   if (pre != NC_NONE && !out) return -3;
   const int has = sp != nullptr;
   if (has && src_f32 && S < 1) return -4;
