@@ -2574,7 +2574,7 @@ def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tens
     _check(lib().la_mamba2(int(f32), src.data_ptr(), T, nseq, H, P, N, G, taps, ssm_state.shape[0], conv_w.data_ptr(),
                            _ptr(conv_b), dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), norm_w.data_ptr(),
                            int(norm_groups), float(eps), pos.data_ptr(), cu_q.data_ptr(), sslots.data_ptr(),
-                           conv_state.data_ptr(), ssm_state.data_ptr(), int(T == nseq), xs.data_ptr(), cb.data_ptr(),
+                           conv_state.data_ptr(), ssm_state.data_ptr(), int(T == nseq and max_rows == 1), xs.data_ptr(), cb.data_ptr(),
                            dtd.data_ptr(), o.data_ptr(), out.data_ptr(), _ptr(seg), max_rows, _stream()), "la_mamba2")
     return out
 

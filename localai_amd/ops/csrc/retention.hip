@@ -17,6 +17,11 @@
 // is a chain of dependent steps, so it is the number of resident waves that hides its latencies.  A
 // decode batch is the same launch with one-token portions: it then streams each state once, which is
 // its memory bound.  retention_out_kernel: the per-head unit norm and the gate.
+//
+// The scan also serves recurrences of the same shape whose decay changes from token to token and
+// whose q / k rows are shared by groups of heads (state-space mixers, mamba2.hip):
+//   S_t = a_(t,h) S_(t-1) + k_(t,g) (s_(t,h) v_(t,h))^T,   o_t = S_t^T q_(t,g)
+// with a (tok_dec) and s (tok_vs) fp32 per (token, head) and Gqk groups; la::decay_scan_f32 is that entry.
 #include "common.h"
 
 namespace la {
@@ -60,16 +65,17 @@ __global__ __launch_bounds__(256) void retention_rot_kernel(const AT* __restrict
 
 template <typename AT, int R, int C, bool EMIT>
 __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
-    const AT* __restrict__ src, int ld, const float* __restrict__ qk, int H, int Dk, int Dv, const int* __restrict__ pos,
-    const int* __restrict__ cu_q, const int* __restrict__ sslots, float* __restrict__ state,
-    const float* __restrict__ decay, float* __restrict__ o, int P, int mode, int L, int maxseg,
-    float* __restrict__ seg_state) {
+    const AT* __restrict__ src, int ld, long vcol0, const float* __restrict__ qk, int H, int Gqk, int Dk, int Dv,
+    const int* __restrict__ pos, const int* __restrict__ cu_q, const int* __restrict__ sslots, float* __restrict__ state,
+    const float* __restrict__ decay, const float* __restrict__ tok_dec, const float* __restrict__ tok_vs, int ldtok,
+    float* __restrict__ o, int P, int mode, int L, int maxseg, float* __restrict__ seg_state) {
   extern __shared__ float lds[];
   const int DkP = P * R;                 // padded key width (rows beyond Dk hold zeros)
   const int cpw = RT_NT / P * C;         // value columns of this workgroup
   float* qs = lds;                       // [TC][DkP]
   float* ks = qs + RT_TC * DkP;          // [TC][DkP]
   float* vs = ks + RT_TC * DkP;          // [TC][cpw]
+  float* dsh = vs + RT_TC * cpw;         // [TC] decay of every staged token (per-token decays)
   const int h = blockIdx.y, c0 = blockIdx.z * cpw;
   const int tid = threadIdx.x, part = tid % P, cg = tid / P, cb = c0 + cg * C;   // this thread's first column
   // mode RT_WHOLE: a workgroup scans a whole portion, slot state in and out.  Segmented portions:
@@ -98,7 +104,8 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
     st = seg_state + (((long)seg * H + h) * Dv + cb) * Dk;
     zero = mode == RT_LOCAL;
   }
-  const float dec = decay[h];
+  const float dec_h = decay ? decay[h] : 1.f;
+  const int g = h / (H / Gqk);           // q / k rows are shared by the heads of a group
   float S[C][R];
 #pragma unroll
   for (int ci = 0; ci < C; ++ci)
@@ -107,7 +114,7 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
       const int r = j * P + part;
       S[ci][j] = (st && !zero && r < Dk && cb + ci < Dv) ? st[(long)ci * Dk + r] : 0.f;
     }
-  const long vcol = 2L * H * Dk + (long)h * Dv;
+  const long vcol = vcol0 + (long)h * Dv;
   for (int t0 = a; t0 < b; t0 += RT_TC) {
     const int n = min(RT_TC, b - t0);
     __syncthreads();
@@ -115,19 +122,23 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
       const int tt = e / DkP, d = e - tt * DkP;
       float qv = 0.f, kv = 0.f;
       if (d < Dk) {
-        const float* row = qk + ((long)(t0 + tt) * 2 * H + h) * Dk + d;
+        const float* row = qk + ((long)(t0 + tt) * 2 * Gqk + g) * Dk + d;
         if (EMIT) qv = row[0];
-        kv = row[(long)H * Dk];
+        kv = row[(long)Gqk * Dk];
       }
       if (EMIT) qs[e] = qv;
       ks[e] = kv;
     }
     for (int e = tid; e < n * cpw; e += RT_NT) {
       const int tt = e / cpw, cc = e - tt * cpw;
-      vs[e] = (c0 + cc < Dv) ? (float)src[(long)(t0 + tt) * ld + vcol + c0 + cc] : 0.f;
+      float v = (c0 + cc < Dv) ? (float)src[(long)(t0 + tt) * ld + vcol + c0 + cc] : 0.f;
+      if (tok_vs) v *= tok_vs[(long)(t0 + tt) * ldtok + h];
+      vs[e] = v;
     }
+    if (tok_dec && tid < n) dsh[tid] = tok_dec[(long)(t0 + tid) * ldtok + h];
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
+      const float dec = tok_dec ? dsh[tt] : dec_h;
       float vv[C], acc[C];
 #pragma unroll
       for (int ci = 0; ci < C; ++ci) {
@@ -172,8 +183,9 @@ __global__ __launch_bounds__(RT_NT) void retention_scan_kernel(
 // A thread per state element of a (sequence, head).
 __global__ __launch_bounds__(256) void retention_join_kernel(const int* __restrict__ pos, const int* __restrict__ cu_q,
                                                              const int* __restrict__ sslots, float* __restrict__ state,
-                                                             const float* __restrict__ decay, int H, long per_head,
-                                                             int L, float* __restrict__ seg_state) {
+                                                             const float* __restrict__ decay,
+                                                             const float* __restrict__ tok_dec, int ldtok, int H,
+                                                             long per_head, int L, float* __restrict__ seg_state) {
   const int seq = blockIdx.x, h = blockIdx.y;
   const long e = (long)blockIdx.z * 256 + threadIdx.x;
   if (e >= per_head) return;
@@ -184,13 +196,20 @@ __global__ __launch_bounds__(256) void retention_join_kernel(const int* __restri
   const int slot = sslots[seq];
   float* st = slot >= 0 ? state + ((long)slot * H + h) * per_head + e : nullptr;
   float S = (st && pos[a] != 0) ? *st : 0.f;
-  const float dec = decay[h], decL = powf(dec, (float)L);
+  const float dec = decay ? decay[h] : 1.f, decL = powf(dec, (float)L);
   for (int s = 0; s * L < n; ++s) {
     const int len = min(L, n - s * L);
     float* p = seg_state + ((long)(seg + s) * H + h) * per_head + e;
     const float local = *p;
     *p = S;
-    S = fmaf(len == L ? decL : powf(dec, (float)len), S, local);
+    float dseg;
+    if (tok_dec) {        // the segment's decays multiplied in token order, as the scan applies them
+      dseg = 1.f;
+      for (int t = 0; t < len; ++t) dseg *= tok_dec[(long)(a + s * L + t) * ldtok + h];
+    } else {
+      dseg = len == L ? decL : powf(dec, (float)len);
+    }
+    S = fmaf(dseg, S, local);
   }
   if (st) *st = S;
 }
@@ -217,16 +236,12 @@ __global__ __launch_bounds__(256) void retention_out_kernel(const float* __restr
   }
 }
 
+// The scan over prepared rows: v from src (row stride ld, head h at column vcol0 + h Dv), q | k rows
+// fp32 [T][2][Gqk][Dk], a fixed decay per head or tok_dec / tok_vs per (token, head) (row stride ldtok).
 template <typename AT>
-static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, int Dv, const int* pos, const int* cu_q,
-                       const int* sslots, float* state, const float* decay, const float* freqs, float mag, int rot,
-                       float* qk, float* o, float* seg, int max_rows, hipStream_t st) {
-  const float kscale = 1.f / sqrtf((float)Dk);
-  {
-    const long total = (long)T * H * (Dk - (rot >> 1));
-    hipLaunchKernelGGL(retention_rot_kernel<AT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src, ld, H, Dk, pos,
-                       freqs, mag, rot, kscale, qk, total);
-  }
+static int scan_core(const AT* src, int ld, long vcol0, int T, int nseq, int H, int Gqk, int Dk, int Dv, const int* pos,
+                     const int* cu_q, const int* sslots, float* state, const float* decay, const float* tok_dec,
+                     const float* tok_vs, int ldtok, const float* qk, float* o, float* seg, int max_rows, hipStream_t st) {
   // long batches of portions are cut into segments of RT_SEG rows scanned in parallel (two scans and a
   // join instead of one chain of T dependent steps); seg: [T / RT_SEG + nseq][H][Dv][Dk] fp32
   // (max_rows: the longest portion of the batch, known to the host; the grid holds that many segments a sequence)
@@ -247,13 +262,14 @@ static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, in
   const int nz = (Dv + cpw - 1) / cpw;
 #define LA_RT_LAUNCH(RR, CC, EM, MODE, GX)                                                                            \
   {                                                                                                                   \
-    const size_t shm = (size_t)(2 * RT_TC * P * RR + RT_TC * cpw) * sizeof(float);                                    \
+    const size_t shm = (size_t)(2 * RT_TC * P * RR + RT_TC * cpw + RT_TC) * sizeof(float);                            \
     if (shm > 150 * 1024) return -6;                                                                                  \
     if (shm > 48 * 1024)                                                                                              \
       (void)hipFuncSetAttribute((const void*)retention_scan_kernel<AT, RR, CC, EM>,                                   \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                                \
     hipLaunchKernelGGL((retention_scan_kernel<AT, RR, CC, EM>), dim3(GX, H, nz), dim3(RT_NT), shm, st, src, ld,       \
-                       (const float*)qk, H, Dk, Dv, pos, cu_q, sslots, state, decay, o, P, MODE, RT_SEG, maxseg, seg);  \
+                       vcol0, (const float*)qk, H, Gqk, Dk, Dv, pos, cu_q, sslots, state, decay, tok_dec, tok_vs,     \
+                       ldtok, o, P, MODE, RT_SEG, maxseg, seg);                                                       \
   }
 #define LA_RT_R(CC, EM, MODE, GX)                                                                                     \
   {                                                                                                                   \
@@ -276,12 +292,34 @@ static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, in
   LA_RT_SCAN(false, RT_LOCAL, nseq * maxseg)
   const long per_head = (long)Dv * Dk;
   hipLaunchKernelGGL(retention_join_kernel, dim3(nseq, H, (unsigned)((per_head + 255) / 256)), dim3(256), 0, st, pos, cu_q,
-                     sslots, state, decay, H, per_head, RT_SEG, seg);
+                     sslots, state, decay, tok_dec, ldtok, H, per_head, RT_SEG, seg);
   LA_RT_SCAN(true, RT_FINAL, nseq * maxseg)
 #undef LA_RT_SCAN
 #undef LA_RT_R
 #undef LA_RT_LAUNCH
   return (int)hipGetLastError();
+}
+
+template <typename AT>
+static int launch_scan(const AT* src, int ld, int T, int nseq, int H, int Dk, int Dv, const int* pos, const int* cu_q,
+                       const int* sslots, float* state, const float* decay, const float* freqs, float mag, int rot,
+                       float* qk, float* o, float* seg, int max_rows, hipStream_t st) {
+  const float kscale = 1.f / sqrtf((float)Dk);
+  const long total = (long)T * H * (Dk - (rot >> 1));
+  hipLaunchKernelGGL(retention_rot_kernel<AT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src, ld, H, Dk, pos,
+                     freqs, mag, rot, kscale, qk, total);
+  return scan_core<AT>(src, ld, 2L * H * Dk, T, nseq, H, H, Dk, Dv, pos, cu_q, sslots, state, decay, nullptr, nullptr, 0,
+                       qk, o, seg, max_rows, st);
+}
+
+// Scan with per-token decays and value scales over fp32 rows (see the head of this file); seg as in
+// la_retention ([T / RT_SEG + nseq][H][Dv][Dk] fp32, or null: whole portions only).
+int decay_scan_f32(const float* v, int ldv, const float* qk, int T, int nseq, int H, int Gqk, int Dk, int Dv,
+                   const int* pos, const int* cu_q, const int* sslots, float* state, const float* tok_dec,
+                   const float* tok_vs, int ldtok, float* o, float* seg, int max_rows, hipStream_t st) {
+  if (T <= 0 || nseq <= 0 || H <= 0 || Gqk <= 0 || H % Gqk || Dk <= 0 || Dv <= 0 || !tok_dec || ldtok < H) return -1;
+  return scan_core<float>(v, ldv, 0L, T, nseq, H, Gqk, Dk, Dv, pos, cu_q, sslots, state, nullptr, tok_dec, tok_vs, ldtok,
+                          qk, o, seg, max_rows > 0 ? max_rows : T, st);
 }
 
 }  // namespace la

@@ -10,6 +10,11 @@
 //   latent_kv:   row [c (rank) | r (rot)]:  c / sqrt(mean c^2 + eps) * w and the rotated r are stored
 //                as ONE row of a one-head K pool, [blocks][1][BS][rank + rot]: key and value at once.
 //
+//   qk_norm_pages: no rotation: every query and key head divided by its root mean square (fp32,
+//                no weight), queries times a temperature 1 + coef ln(floor((pos + 1) / every) + 1);
+//                K / V appended as above.  A wave per head.
+//   sinusoid_add: additive positions on the fp32 stream, column 2i += sin(pos f_i), 2i + 1 += cos.
+//
 // A workgroup per token; the token's cos / sin are computed once into LDS.
 #include "common.h"
 
@@ -107,7 +112,82 @@ __global__ __launch_bounds__(RP_NT) void latent_kv_kernel(const AT* __restrict__
   (void)BS;
 }
 
+// row [q (H x Dq) | k (G x Dk) | v (G x Dv)] with row stride ld: unit-RMS q (times the position's
+// temperature) -> q_out, unit-RMS k and v -> pages.  Wave w of the workgroup takes heads w, w + 4, ...
+template <typename AT>
+__global__ __launch_bounds__(RP_NT) void qk_norm_pages_kernel(const AT* __restrict__ src, long ld, int H, int Dq, int G,
+                                                              int Dk, int Dv, const int* __restrict__ pos,
+                                                              const int* __restrict__ slots, float eps, float coef,
+                                                              int every, AT* __restrict__ q_out, AT* __restrict__ kc,
+                                                              AT* __restrict__ vc, int BS) {
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int Cq = H * Dq, Ck = G * Dk, Cv = G * Dv;
+  const AT* row = src + (long)t * ld;
+  float tau = 1.f;
+  if (every > 0) tau = 1.f + coef * logf((float)((pos[t] + 1) / every + 1));
+  const int slot = G ? slots[t] : -1;
+  const int blk = slot >= 0 ? slot / BS : 0, off = slot >= 0 ? slot - blk * BS : 0;
+  for (int u = wave; u < H + G; u += RP_NT / 64) {
+    const bool isq = u < H;
+    if (!isq && slot < 0) continue;
+    const int n = isq ? Dq : Dk;
+    const AT* x = isq ? row + (long)u * Dq : row + Cq + (long)(u - H) * Dk;
+    float ss = 0.f;
+    for (int d = lane; d < n; d += 64) {
+      const float v = (float)x[d];
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    const float f = (1.f / sqrtf(ss / (float)n + eps)) * (isq ? tau : 1.f);
+    AT* dst = isq ? q_out + (long)t * Cq + (long)u * Dq : kc + (((long)blk * G + (u - H)) * BS + off) * Dk;
+    for (int d = lane; d < n; d += 64) dst[d] = (AT)((float)x[d] * f);
+  }
+  if (slot < 0) return;
+  for (int e = tid; e < Cv; e += RP_NT) {
+    const int g = e / Dv, d = e - g * Dv;
+    vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)] = row[Cq + Ck + e];
+  }
+}
+
+__global__ __launch_bounds__(256) void sinusoid_add_kernel(float* __restrict__ res, int D, const int* __restrict__ pos,
+                                                           const float* __restrict__ freqs) {
+  const int t = blockIdx.x;
+  const float p = (float)pos[t];
+  for (int i = threadIdx.x; 2 * i < D; i += 256) {
+    const float a = p * freqs[i];
+    float* r = res + (long)t * D + 2 * i;
+    r[0] += sinf(a);
+    if (2 * i + 1 < D) r[1] += cosf(a);
+  }
+}
+
 }  // namespace la
+
+extern "C" int la_qk_norm_pages(int f32, const void* src, int ld, int T, int H, int Dq, int G, int Dk, int Dv,
+                                const void* pos, const void* slots, float eps, float coef, int every, void* q_out,
+                                void* kc, void* vc, int BS, void* stream) {
+  using namespace la;
+  if (T <= 0 || H <= 0 || Dq <= 0 || G < 0 || every < 0 || ld < H * Dq + G * Dk + G * Dv) return -1;
+  if (G && (Dk <= 0 || Dv <= 0 || !kc || !vc || !slots || BS <= 0 || (BS & 7))) return -2;
+  if (!src || !pos || !q_out) return -3;
+  if (f32)
+    hipLaunchKernelGGL(qk_norm_pages_kernel<float>, dim3(T), dim3(RP_NT), 0, (hipStream_t)stream, (const float*)src, (long)ld,
+                       H, Dq, G, Dk, Dv, (const int*)pos, (const int*)slots, eps, coef, every, (float*)q_out, (float*)kc,
+                       (float*)vc, BS);
+  else
+    hipLaunchKernelGGL(qk_norm_pages_kernel<bf16>, dim3(T), dim3(RP_NT), 0, (hipStream_t)stream, (const bf16*)src, (long)ld,
+                       H, Dq, G, Dk, Dv, (const int*)pos, (const int*)slots, eps, coef, every, (bf16*)q_out, (bf16*)kc,
+                       (bf16*)vc, BS);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_sinusoid_add(void* res, int T, int D, const void* pos, const void* freqs, void* stream) {
+  using namespace la;
+  if (T <= 0 || D <= 0 || !res || !pos || !freqs) return -1;
+  hipLaunchKernelGGL(sinusoid_add_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, (float*)res, D, (const int*)pos,
+                     (const float*)freqs);
+  return (int)hipGetLastError();
+}
 
 extern "C" int la_rope_pages(int f32, const void* src, int T, int H, int Dq, int G, int Dk, int Dv, const void* pos,
                              const void* slots, const void* freqs, float mag, int rot, int q_off, int interleaved,
