@@ -1429,3 +1429,84 @@ def write_dadizen(out_dir: str, width: int = 256, kinds=("attention", "latent_at
         json.dump(cfg, f)
     save_file(W, os.path.join(out_dir, "model.safetensors"))
     return out_dir
+
+
+def write_vinozen(out_dir: str, width: int = 256, kinds=("attention", "mamba2"), heads: int = 4, kv_heads: int = 2,
+                  dim: int = 64, vdim: int = 64, bias_rows: int = 32, bias_max: int = 128, temp_every: int = 256,
+                  share_kv: bool = False, m_heads: int = 8, m_vdim: int = 64, m_state: int = 64, m_groups: int = 1,
+                  conv: int = 4, norm_groups: int = 1, ff: int = 1024, experts: int = 0, top: int = 2,
+                  expert_ff: int = 256, shared_ff: int = 0, side_dim: int = 32, vocab: int = 32000, seed: int = 0) -> str:
+    """Random-init Vinozen checkpoint directory (config.json + model.safetensors, bf16): one layer
+    per entry of `kinds` (the mixer types), all of the given sizes; share_kv: attention layers after
+    the first attend over the first one's pages; experts > 0: routed clamped experts (plus a shared
+    one of width shared_ff) instead of the dense SwiGLU feed-forward; a token side input of
+    `side_dim` columns (0: none).  Benchmarks and smoke runs; the weights mean nothing."""
+    import json
+
+    import torch
+    from safetensors.torch import save_file
+    os.makedirs(out_dir, exist_ok=True)
+    g = torch.Generator().manual_seed(seed)
+    D, n = width, len(kinds)
+
+    def rnd(*shape, s):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * s).to(torch.bfloat16)
+
+    def lin(a, b):
+        return rnd(a, b, s=b ** -0.5)
+
+    def norm(k):
+        return (1.0 + rnd(k, s=0.05).float()).to(torch.bfloat16)
+
+    W = {"embed": rnd(vocab, D, s=0.05), "final.norm": norm(D)}
+    if side_dim:
+        W["side.embed"] = rnd(vocab, n * side_dim, s=1.0)
+    layers, first_attn = [], -1
+    for i, kind in enumerate(kinds):
+        p = f"l{i}."
+        W[p + "norm1"], W[p + "norm2"] = norm(D), norm(D)
+        if kind == "attention":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5 * 4.0,
+                 "bias_max": bias_max, "q_temp": {"coef": 0.1, "every": temp_every}}
+            W[p + "mix.q"] = lin(heads * dim, D)
+            if share_kv and first_attn >= 0:
+                m["kv_from"] = first_attn
+            else:
+                W[p + "mix.k"], W[p + "mix.v"] = lin(kv_heads * dim, D), lin(kv_heads * vdim, D)
+                first_attn = i if first_attn < 0 else first_attn
+            W[p + "mix.rel"], W[p + "mix.sink"] = rnd(bias_rows, heads, s=0.5), rnd(heads, s=0.5)
+            W[p + "mix.o"] = lin(D, heads * vdim)
+        elif kind == "mamba2":
+            m = {"heads": m_heads, "vdim": m_vdim, "state": m_state, "groups": m_groups, "conv": conv, "norm_groups": norm_groups}
+            inner, gn = m_heads * m_vdim, m_groups * m_state
+            W[p + "mix.in"] = lin(2 * inner + 2 * gn + m_heads, D)
+            W[p + "mix.conv"], W[p + "mix.conv.b"] = rnd(inner + 2 * gn, conv, s=0.4), rnd(inner + 2 * gn, s=0.1)
+            W[p + "mix.dt_bias"] = (rnd(m_heads, s=0.5).float() - 3.0).to(torch.bfloat16)
+            W[p + "mix.A_log"], W[p + "mix.D"] = rnd(m_heads, s=0.5), (1.0 + rnd(m_heads, s=0.1).float()).to(torch.bfloat16)
+            W[p + "mix.norm"], W[p + "mix.o"] = norm(inner), lin(D, inner)
+        else:
+            raise ValueError(f"unknown mixer kind {kind!r}")
+        if experts:
+            f = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+            for e in range(experts):
+                q = p + f"mlp.e{e}."
+                W[q + "gate"], W[q + "up"], W[q + "down"] = lin(expert_ff, D), lin(expert_ff, D), lin(D, expert_ff)
+            W[p + "mlp.router"], W[p + "mlp.router.b"] = lin(experts, D), rnd(experts, s=0.1)
+            if shared_ff:
+                f["shared"] = {"ff": shared_ff, "limit": 7.0}
+                q = p + "mlp.shared."
+                W[q + "gate"], W[q + "up"], W[q + "down"] = lin(shared_ff, D), lin(shared_ff, D), lin(D, shared_ff)
+        else:
+            f = {"kind": "dense", "ff": ff}
+            W[p + "mlp.gate"], W[p + "mlp.up"], W[p + "mlp.down"] = lin(ff, D), lin(ff, D), lin(D, ff)
+        if side_dim:
+            W[p + "side.gate"], W[p + "side.proj"], W[p + "side.norm"] = lin(side_dim, D), lin(D, side_dim), rnd(D, s=0.1)
+        layers.append({"type": kind, "mixer": m, "mlp": f})
+    cfg = {"architecture": "Vinozen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 20.0},
+           "layers": layers}
+    if side_dim:
+        cfg["token_side"] = {"dim": side_dim}
+    with open(os.path.join(out_dir, "config.json"), "w") as f_:
+        json.dump(cfg, f_)
+    save_file(W, os.path.join(out_dir, "model.safetensors"))
+    return out_dir

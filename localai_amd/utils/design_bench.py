@@ -3,7 +3,9 @@ layer sizes (bench.py --design-compare): random weights, bf16, one GPU.
 
 For each size two-layer models are built -- Suganex: dense feed-forwards (beside a llama
 checkpoint) and routed experts (beside a Mixtral-style checkpoint); Dadizen: one model per mixer
-kind (windowed attention, latent attention, retention) beside the llama checkpoint -- all stored as
+kind (windowed attention, latent attention, retention) beside the llama checkpoint; Vinozen:
+attention with a dense feed-forward, attention with routed experts, the state-space mixer, beside
+the llama and Mixtral-style checkpoints -- all stored as
 dense bf16 weights so every GEMM takes the same library path, and each is timed through its engine's own
 batch construction (native scheduler, paged KV pool, state slots) and `model.forward`:
   prefill: `n_seq` prompts of `prompt` tokens in one batch, tokens/s;
@@ -65,6 +67,28 @@ def _dadizen_models(size: str, cache: str) -> Dict[str, str]:
                                 side_dim=s["dim"], vocab=VOCAB, **kw)
         out[f"dadizen-{kind}"] = p
     out["llama-dense"] = _llama(size, cache)
+    return out
+
+
+def _vinozen_models(size: str, cache: str) -> Dict[str, str]:
+    """Two equal layers each: attention with a dense feed-forward (beside the llama checkpoint), attention
+    with routed experts and no shared expert (beside the Mixtral-style checkpoint, equal expert count
+    and widths), the state-space mixer with a dense feed-forward (inner width twice the model width
+    in heads of 64 channels, state 128, one group, 4 taps: the usual proportions of such layers)."""
+    from ..models import synth
+    s = SIZES[size]
+    out = {}
+    for kind in ("attention-dense", "attention-moe", "mamba2-dense"):
+        p = os.path.join(cache, f"vinozen-{size}-{kind}")
+        mix, f = kind.split("-")
+        if not os.path.exists(os.path.join(p, "model.safetensors")):
+            synth.write_vinozen(p, width=s["width"], kinds=(mix, mix), heads=s["heads"], kv_heads=s["kv"], dim=s["dim"],
+                                vdim=s["dim"], m_heads=2 * s["width"] // 64, m_vdim=64, m_state=128, ff=s["ff"],
+                                experts=s["experts"] if f == "moe" else 0, top=s["top"], expert_ff=s["eff"],
+                                side_dim=s["dim"], vocab=VOCAB)
+        out[f"vinozen-{kind}"] = p
+    out["llama-dense"] = _llama(size, cache)
+    out["mixtral-moe"] = _llama(size, cache, moe=True)
     return out
 
 
@@ -174,15 +198,15 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
 
 def run(design: str, sizes: List[str], cache: str, n_seq: int = 4, prompt: int = 2048, batch: int = 64,
         context: int = 1536, iters: int = 5) -> dict:
-    if design not in ("suganex", "dadizen"):
-        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex, dadizen)")
+    if design not in ("suganex", "dadizen", "vinozen"):
+        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex, dadizen, vinozen)")
     os.makedirs(cache, exist_ok=True)
     res = {"design": design, "dtype": "bf16", "data": "synthetic", "layers": 2,
            "workload": {"prefill": f"{n_seq} x {prompt} tokens", "decode": f"batch {batch} at context {context}"},
            "sizes": {}}
     for size in sizes:
         t0 = time.time()
-        paths = _models(size, cache) if design == "suganex" else _dadizen_models(size, cache)
+        paths = {"suganex": _models, "dadizen": _dadizen_models, "vinozen": _vinozen_models}[design](size, cache)
         row = {}
         for name, p in paths.items():
             row[name] = {k: round(v, 3 if k.endswith("ms") else 1)
