@@ -153,6 +153,7 @@ class _Layer:
     bias: Optional[torch.Tensor] = None          # attention: distance-bias table fp32 [bias_max + 1, H]
     sink: Optional[torch.Tensor] = None          # fp32 [H]
     conv: Optional[torch.Tensor] = None          # mamba2: fp32 [C, taps]
+    conv_t: Optional[torch.Tensor] = None        # the same tap-major, [taps, C] (the vectorised kernel's layout)
     conv_b: Optional[torch.Tensor] = None
     dt_bias: Optional[torch.Tensor] = None
     a_log: Optional[torch.Tensor] = None
@@ -267,6 +268,7 @@ class VinozenModel:
         L = _Layer(self._f32(p + "norm1", (D,)), self._qw(sh(p + "mix.in", (2 * inner + 2 * GN + H, D))),
                    self._qw(sh(p + "mix.o", (D, inner))))
         L.conv = self._f32(p + "mix.conv", (C, m.taps))
+        L.conv_t = L.conv.t().contiguous()
         L.conv_b = self._f32(p + "mix.conv.b", (C,))
         L.dt_bias, L.a_log, L.d_skip = (self._f32(p + n, (H,)) for n in ("mix.dt_bias", "mix.A_log", "mix.D"))
         L.mix_norm = self._f32(p + "mix.norm", (inner,))
@@ -320,7 +322,21 @@ class VinozenModel:
         return KVCache.layered(self._specs(), num_blocks, block_size, self.device, self.dtype, state_slots)
 
     def decode_workspace(self, Bp: int, ctx: int, block_size: int):
-        return None
+        """Split-KV buffers of the decode attention kernel per (heads, kv heads, width) of the layers it serves."""
+        out = {}
+        for m in self.hp.mixers:
+            if m.kind == "attention" and self._decode_kernel_ok(m, block_size):
+                key = (m.heads, m.kv_heads, m.dim)
+                if key not in out:
+                    out[key] = ops.decode_workspace(Bp, m.heads, m.kv_heads, m.dim, ctx, self.device, block_size)
+        return out or None
+
+    def _decode_kernel_ok(self, m: MixSpec, block_size: int) -> bool:
+        """Decode batches of this layer on the framework's split-KV decode attention kernel (the llama
+        families'): bf16, equal key and value widths it is instantiated for; it takes the bias table and the sink."""
+        return (not self.f32 and self.device.type == "cuda" and m.dim == m.vdim and m.dim in (64, 80, 96, 128, 192, 256)
+                and m.heads // m.kv_heads <= 16 and block_size % 16 == 0 and (128 % block_size == 0 or block_size % 128 == 0)
+                and ops._has("la_attn_decode"))
 
     def prefill_tiles(self, q_lens, device):
         """(16-row work tiles of the leading prompt portions for ops.attn_mix, rows they cover)."""
@@ -399,13 +415,17 @@ class VinozenModel:
             y = y + self._dense(self._unit(xn, L.shared, f.shared_ff, f.shared_limit)).float()
         return y
 
-    def _attention(self, L: _Layer, m: MixSpec, i: int, xn, fb, kv, row_seq, cu_q, tiles, tile_rows, splits):
+    def _attention(self, L: _Layer, m: MixSpec, i: int, xn, fb, kv, row_seq, cu_q, tiles, tile_rows, splits, ws=None):
         proj = self._dense(ops.linear(xn, L.win))
         own = m.kv_from < 0
         src = i if own else m.kv_from
         q = ops.qk_norm_pages(proj, m.heads, m.dim, m.kv_heads if own else 0, m.dim, m.vdim, fb.pos, fb.slots,
                               self.hp.norm_eps, m.temp_coef, m.temp_every, kv.k[src] if own else None,
                               kv.v[src] if own else None)
+        if fb.decode and fb.seq_lens is not None and self._decode_kernel_ok(m, kv.block_size):
+            T = q.shape[0]
+            return ops.attn_decode(q.view(T, m.heads, m.dim), kv.k[src], kv.v[src], fb.block_tables, fb.seq_lens, m.scale,
+                                   fb.max_len, workspace=ws, dist_bias=L.bias, sink=L.sink).view(T, m.heads * m.vdim)
         return ops.attn_mix(q, kv.k[src], kv.v[src], row_seq, fb.pos, fb.block_tables, m.heads, m.scale,
                             tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits, dist_bias=L.bias, sink=L.sink)
 
@@ -414,7 +434,7 @@ class VinozenModel:
         conv_state, ssm_state = kv.state[i]
         return ops.mamba2(proj, m.heads, m.vdim, m.state, m.groups, L.conv, L.conv_b, L.dt_bias, L.a_log, L.d_skip,
                           L.mix_norm, m.norm_groups, self.hp.norm_eps, fb.pos, cu_q, fb.sslots, conv_state, ssm_state,
-                          max_rows=1 if fb.decode else fb.max_q)
+                          max_rows=1 if fb.decode else fb.max_q, conv_wt=L.conv_t)
 
     def forward(self, fb: ForwardBatch, kv: KVCache, attn_workspace=None, return_hidden: bool = False,
                 local_logits: bool = False, layer_out: Optional[list] = None) -> torch.Tensor:
@@ -448,7 +468,8 @@ class VinozenModel:
         xn = nc(None, None, cast)        # the sublayers read the stream itself
         for i, (L, m, f) in enumerate(zip(self.layers, hp.mixers, hp.mlps)):
             if m.kind == "attention":
-                a = self._attention(L, m, i, xn, fb, kv, row_seq, cu_q, tiles, tile_rows, splits)
+                ws = attn_workspace.get((m.heads, m.kv_heads, m.dim)) if isinstance(attn_workspace, dict) else None
+                a = self._attention(L, m, i, xn, fb, kv, row_seq, cu_q, tiles, tile_rows, splits, ws)
             else:
                 a = self._mamba2(L, m, i, xn, fb, kv, cu_q)
             last = self.out_norm if i + 1 == n else cast       # what the layer's last boundary hands on

@@ -86,7 +86,8 @@ def lib():
             "la_reduce_slabs": [P, LNG, I, P, I, I, P, P, P],
             "la_embed": [I, P, P, P, P, I, I, P, I, P, F, P],
             "la_dequant": [I, P, P, P, P, I, I, P, P],
-            "la_attn_decode": [P, P, P, P, I, P, I, I, I, I, I, F, I, I, P, P, P, P, P, LNG, I, P, P, P, P, F, I, I, P],
+            "la_attn_decode": [P, P, P, P, I, P, I, I, I, I, I, F, I, I, P, P, P, P, P, LNG, I, P, P, P, P, F, I, I, P, I, P,
+                               P],
             "la_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, F, P, F, I, P],
             "la_sample": [P, LNG, I, I, P, P, P, P, P],
             "la_penalties": [P, LNG, I, P, I, P, P, I, P, P],
@@ -128,7 +129,7 @@ def lib():
             "la_moe_pairs": [I, P, P, P, P, P, P, I, I, I, I, I, P, P, I, F, F, P],
             "la_sinusoid_add": [P, I, I, P, P, P],
             "la_qk_norm_pages": [I, P, I, I, I, I, I, I, I, P, P, F, F, I, P, P, P, I, P],
-            "la_mamba2": [I, P, I, I, I, I, I, I, I, I, P, P, P, P, P, P, I, F, P, P, P, P, P, I, P, P, P, P, P, P, I,
+            "la_mamba2": [I, P, I, I, I, I, I, I, I, I, P, P, P, P, P, P, P, I, F, P, P, P, P, P, I, P, P, P, P, P, P, I,
                           P],
             "la_attn_latent": [P, P, P, P, P, I, I, I, I, I, I, F, I, P, I, P, I, P, P, P],
             "la_norm_chain": [P, I, I, P, I, LNG, I, I, F, P, P, F, P, I, I, F, P, P, P, I, P],
@@ -1525,16 +1526,24 @@ def decode_workspace(B: int, Hq: int, Hkv: int, Dh: int, max_len: int, device, b
 def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                 seq_lens: torch.Tensor, scale: float, max_seq_len: int, out: Optional[torch.Tensor] = None,
                 workspace: Optional[Tuple[torch.Tensor, ...]] = None, softcap: float = 0.0,
-                window: int = 0) -> torch.Tensor:
+                window: int = 0, dist_bias: Optional[torch.Tensor] = None,
+                sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [B,Hq,Dh] bf16; K cache [nblk,Hkv,BS,Dh]; V cache (grouped-transposed pages)
     [nblk,Hkv,BS/8,Dh,8]; block_tables [B,maxb] i32; seq_lens [B] i32.  softcap > 0: scores
-    softcap * tanh(s / softcap); window > 0: only the last `window` keys are attended (Gemma-2)."""
+    softcap * tanh(s / softcap); window > 0: only the last `window` keys are attended (Gemma-2).
+    dist_bias (fp32 [N, Hq]) / sink (fp32 [Hq]): a bias per distance and head (constant from row
+    N - 1 on) and a logit without key or value in the softmax denominator, as in attn_mix."""
     B, Hq, Dh = q.shape
     nblk, Hkv, BS, Dh2 = k_cache.shape
     if Dh2 != Dh or Hq % Hkv or tuple(v_cache.shape) != (nblk, Hkv, BS // 8, Dh, 8):
         raise ValueError("attn_decode: head/cache shape mismatch")
     if not q.is_cuda:
+        if dist_bias is not None or sink is not None:
+            raise ValueError("attn_decode: distance bias and sink have no CPU path here (attn_mix has)")
         return _attn_ref_decode(q, k_cache, v_cache, block_tables, seq_lens, scale, softcap, window)
+    for t in (dist_bias, sink):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda or t.shape[-1] != Hq):
+            raise ValueError("attn_decode: dist_bias [N, Hq] and sink [Hq] are contiguous fp32")
     P, PS = decode_partitions(B, Hkv, max_seq_len, BS)
     if out is None:
         out = torch.empty(B, Hq, Dh, dtype=torch.bfloat16, device=q.device)
@@ -1545,7 +1554,8 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     _check(lib().la_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
                                 block_tables.shape[1], seq_lens.data_ptr(), B, Hq, Hkv, Dh, BS, float(scale), P, PS,
                                 out.data_ptr(), po.data_ptr(), pml.data_ptr(), tk.data_ptr(), None, 0, 0, None, None,
-                                None, None, float(softcap), int(window), _dec_nw(B, Hkv), _stream()),
+                                None, None, float(softcap), int(window), _dec_nw(B, Hkv), _ptr(dist_bias),
+                                dist_bias.shape[0] if dist_bias is not None else 0, _ptr(sink), _stream()),
            "la_attn_decode")
     return out
 
@@ -1590,7 +1600,7 @@ def attn_decode_rope(qkv: Partial, pos: torch.Tensor, slots: torch.Tensor, cos_s
                                 block_tables.shape[1], seq_lens.data_ptr(), T, Hq, Hkv, Dh, BS, float(scale), P, PS,
                                 out.data_ptr(), po.data_ptr(), pml.data_ptr(), tk.data_ptr(), a[0], a[1], a[2], a[3],
                                 pos.data_ptr(), slots.data_ptr(), cos_sin.data_ptr(), float(softcap), int(window),
-                                _dec_nw(T, Hkv), _stream()),
+                                _dec_nw(T, Hkv), None, 0, None, _stream()),
            "la_attn_decode(rope)")
     return out
 
@@ -2492,7 +2502,7 @@ def mamba2_states(slots: int, H: int, P: int, N: int, G: int, taps: int, dtype=t
 def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tensor, conv_b: Optional[torch.Tensor],
            dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor, norm_w: torch.Tensor, norm_groups: int,
            eps: float, pos: torch.Tensor, cu_q: torch.Tensor, sslots: torch.Tensor, conv_state: torch.Tensor,
-           ssm_state: torch.Tensor, max_rows: int = 0) -> torch.Tensor:
+           ssm_state: torch.Tensor, max_rows: int = 0, conv_wt: Optional[torch.Tensor] = None) -> torch.Tensor:
     """State-space mixer with a scalar decay per head (state-space duality form) over projection
     rows src [T, 2 H P + 2 G N + H] laid out [z | x | B | C | dt]:
       * x, B, C pass a depthwise causal convolution over time (conv_w [H P + 2 G N, taps] fp32, last
@@ -2505,7 +2515,9 @@ def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tens
     comes from conv_state[sslots[seq]] (the last taps - 1 rows of [x | B | C] before the
     convolution) and ssm_state[sslots[seq]] (fp32), both taken as zero before position 0, and both
     are advanced to the portion's end.  dt, decays, the recurrence, its state and outputs, the gate
-    and the norm are fp32.  Returns [T, H P] in src's dtype."""
+    and the norm are fp32.  conv_wt: conv_w tap-major ([taps, C] fp32), which the vectorised
+    kernel reads (widths that are multiples of 8); made per call when not given.  Returns
+    [T, H P] in src's dtype."""
     T = src.shape[0]
     nseq = cu_q.shape[0] - 1
     inner, GN = H * P, G * N
@@ -2563,6 +2575,10 @@ def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tens
     for t in (conv_w, conv_b, dt_bias, a_log, d_skip, norm_w):
         assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda)
     dev = src.device
+    if conv_wt is None and not (inner % 8 or GN % 8 or H % 8):
+        conv_wt = conv_w.t().contiguous()
+    if conv_wt is not None and (conv_wt.dtype != torch.float32 or tuple(conv_wt.shape) != (taps, C) or not conv_wt.is_contiguous()):
+        raise ValueError("mamba2: conv_wt must be the fp32 [taps, C] transpose of conv_w")
     xs = torch.empty(T, inner, dtype=torch.float32, device=dev)         # convolved x
     cb = torch.empty(T, 2 * GN, dtype=torch.float32, device=dev)        # convolved C | B: the scan's q | k rows
     dtd = torch.empty(T, 2 * H, dtype=torch.float32, device=dev)        # dt | decay per (token, head)
@@ -2572,7 +2588,7 @@ def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tens
     seg = torch.empty((T // RETENTION_SEG + nseq) * H * P * N, dtype=torch.float32, device=dev) \
         if (T >= 8 * RETENTION_SEG and max_rows >= 4 * RETENTION_SEG) else None
     _check(lib().la_mamba2(int(f32), src.data_ptr(), T, nseq, H, P, N, G, taps, ssm_state.shape[0], conv_w.data_ptr(),
-                           _ptr(conv_b), dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), norm_w.data_ptr(),
+                           _ptr(conv_wt), _ptr(conv_b), dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), norm_w.data_ptr(),
                            int(norm_groups), float(eps), pos.data_ptr(), cu_q.data_ptr(), sslots.data_ptr(),
                            conv_state.data_ptr(), ssm_state.data_ptr(), int(T == nseq and max_rows == 1), xs.data_ptr(), cb.data_ptr(),
                            dtd.data_ptr(), o.data_ptr(), out.data_ptr(), _ptr(seg), max_rows, _stream()), "la_mamba2")

@@ -112,6 +112,15 @@ LA_DEV void rope_src_load(const DecRope& R, int b, int col, float (&v)[N]) {
   }
 }
 
+// Score extras of designs without rotation: a bias per distance and head added to the scaled score
+// (table [n][Hq] fp32, constant from row n - 1 on) and a sink logit per head that joins the softmax
+// denominator once, without key or value (counted by wave 0 of the first partition).
+struct DecExtra {
+  const float* bias;
+  int nbias;
+  const float* sink;
+};
+
 // K/V are streamed once per decode step: non-temporal loads (the default) read them 12-14 %
 // faster at batch 256 (5.05 -> 5.70 TB/s at 256 keys, 5.21 -> 5.98 at 384;
 // profiles/r4_attn_decode_nt.md).  VAR bit 0 = ordinary cached loads (A/B only); bit 1 = keys
@@ -122,7 +131,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ seq_lens, int Hkv, int G,
     int BS, float scale_log2, int PS_grid, bf16* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int P, int* __restrict__ tickets, DecRope R, float cap_l2, float cap_mul,
-    int window, int one_part) {
+    int window, int one_part, DecExtra E) {
   constexpr int KC = (DH + 31) / 32;  // 32-wide k chunks of the QK^T product
   constexpr int ND = DH / 16;         // 16-wide d tiles of the PV product
   constexpr int NT = NW * 64;
@@ -240,6 +249,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
   for (int i = 0; i < ND; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
+  const int hq_r = kvh * G + min(r, G - 1);          // this lane's query head (lanes r >= G: padding)
+  if (E.sink && p == 0 && wave == 0) {
+    m = E.sink[hq_r] * 1.4426950408889634f;
+    lsum = g == 0 ? 1.f : 0.f;                        // the lane groups' sums are added up at the end
+  }
 
   // register double buffer up to Dh 128; a Dh-256 tile (Gemma) is 128 VGPRs on its own, so it
   // is loaded at the top of each iteration instead (no prefetch, no spills)
@@ -281,7 +295,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
           const int key = kb + 8 * g + 4 * t + i;
           // Gemma-2 logit soft-capping cap * tanh(s / cap) (cap_l2 = cap * log2 e, 0: off) and
           // sliding-window attention (keys at least `window` positions behind the query masked)
-          const float sv = cap_l2 > 0.f ? cap_l2 * tanhf(acc[i] * cap_mul) : acc[i] * scale_log2;
+          float sv = cap_l2 > 0.f ? cap_l2 * tanhf(acc[i] * cap_mul) : acc[i] * scale_log2;
+          if (E.bias) sv = fmaf(E.bias[(long)min(max(L - 1 - key, 0), E.nbias - 1) * Hq + hq_r], 1.4426950408889634f, sv);
           s[t][i] = (key < kend && key >= wlo) ? sv : -INFINITY;
         }
       }
@@ -631,7 +646,8 @@ extern "C" int la_attn_decode(const void* q, const void* kc, const void* vc, con
                               const int* seq_lens, int B, int Hq, int Hkv, int Dh, int BS, float scale, int P, int PS,
                               void* out, void* part_o, void* part_ml, void* tickets, const void* rope_p,
                               long rope_slab, int rope_S, const void* rope_bias, const int* pos, const int* slots,
-                              const float* cos_sin, float softcap, int window, int nw, void* stream) {
+                              const float* cos_sin, float softcap, int window, int nw, const float* dist_bias,
+                              int nbias, const float* sink, void* stream) {
   // nw bit 8: split even short sequences over the grid's partitions (few sequences: the
   // parallelism is worth the merge); otherwise a sequence of <= DEC_ONE_PART keys is one partition
   const int one_part = (nw & 256) ? 0 : g_dec_one_part;
@@ -644,6 +660,8 @@ extern "C" int la_attn_decode(const void* q, const void* kc, const void* vc, con
   if (rope_p && ((Dh & 31) || !pos || !slots || !cos_sin || rope_S < 0)) return -1;
   if (!rope_p && !q) return -1;
   const la::DecRope R{rope_p, rope_slab, rope_S, (const float*)rope_bias, pos, slots, cos_sin, (Hq + 2 * Hkv) * Dh};
+  if (dist_bias && nbias < 1) return -1;
+  const la::DecExtra E{dist_bias, nbias, sink};
   const int G = Hq / Hkv;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(P, Hkv, B);
@@ -660,7 +678,7 @@ extern "C" int la_attn_decode(const void* q, const void* kc, const void* vc, con
 #define DEC_LAUNCH(D, GT, NW, V)                                                                                  \
   hipLaunchKernelGGL((la::attn_decode_kernel<D, GT, NW, V>), grid, dim3(NW * 64), 0, st, (const bf16*)q,        \
                      (const bf16*)kc, (const bf16*)vc, block_tables, max_blocks, seq_lens, Hkv, G, BS, sl2, PS,  \
-                     (bf16*)out, po, pml, P, tk, R, cap_l2, cap_mul, window, one_part)
+                     (bf16*)out, po, pml, P, tk, R, cap_l2, cap_mul, window, one_part, E)
 #define DEC_NW(D, GT, NW)                                                  \
   do {                                                                     \
     if constexpr (D == 128 && GT == 4 && NW == 1) {                        \

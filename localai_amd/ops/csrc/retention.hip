@@ -29,6 +29,7 @@ namespace la {
 constexpr int RT_NT = 256;
 constexpr int RT_TC = 16;     // tokens staged per chunk
 constexpr int RT_SEG = 128;   // rows per segment of a segmented portion
+constexpr int RT_JOIN_MAXSEG = 1024;   // segments of one portion the join holds decay products for
 enum { RT_WHOLE = 0, RT_LOCAL = 1, RT_FINAL = 2 };
 
 // qk[t][0][h][d] = rotated q, qk[t][1][h][d] = rotated k * kscale (fp32): a thread per (row, head, pair or plain dim)
@@ -188,27 +189,37 @@ __global__ __launch_bounds__(256) void retention_join_kernel(const int* __restri
                                                              long per_head, int L, float* __restrict__ seg_state) {
   const int seq = blockIdx.x, h = blockIdx.y;
   const long e = (long)blockIdx.z * 256 + threadIdx.x;
-  if (e >= per_head) return;
   const int a = cu_q[seq], n = cu_q[seq + 1] - a;
   if (n <= 0) return;
   int seg = 0;
   for (int s2 = 0; s2 < seq; ++s2) seg += (cu_q[s2 + 1] - cu_q[s2] + L - 1) / L;
   const int slot = sslots[seq];
-  float* st = slot >= 0 ? state + ((long)slot * H + h) * per_head + e : nullptr;
+  float* st = (slot >= 0 && e < per_head) ? state + ((long)slot * H + h) * per_head + e : nullptr;
   float S = (st && pos[a] != 0) ? *st : 0.f;
   const float dec = decay ? decay[h] : 1.f, decL = powf(dec, (float)L);
-  for (int s = 0; s * L < n; ++s) {
+  // per-token decays: every segment's product once per workgroup (a wave per segment, two shuffles
+  // deep per 64 tokens), not once per state element
+  __shared__ float sd[RT_JOIN_MAXSEG];
+  const int nsegs = (n + L - 1) / L;
+  if (tok_dec) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int s = wave; s < nsegs; s += 4) {
+      const int len = min(L, n - s * L);
+      float pd = 1.f;
+      for (int t = lane; t < len; t += 64) pd *= tok_dec[(long)(a + s * L + t) * ldtok + h];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) pd *= __shfl_xor(pd, o, 64);
+      if (lane == 0) sd[s] = pd;
+    }
+    __syncthreads();
+  }
+  if (e >= per_head) return;
+  for (int s = 0; s < nsegs; ++s) {
     const int len = min(L, n - s * L);
     float* p = seg_state + ((long)(seg + s) * H + h) * per_head + e;
     const float local = *p;
     *p = S;
-    float dseg;
-    if (tok_dec) {        // the segment's decays multiplied in token order, as the scan applies them
-      dseg = 1.f;
-      for (int t = 0; t < len; ++t) dseg *= tok_dec[(long)(a + s * L + t) * ldtok + h];
-    } else {
-      dseg = len == L ? decL : powf(dec, (float)len);
-    }
+    const float dseg = tok_dec ? sd[s] : (len == L ? decL : powf(dec, (float)len));
     S = fmaf(dseg, S, local);
   }
   if (st) *st = S;
@@ -245,7 +256,8 @@ static int scan_core(const AT* src, int ld, long vcol0, int T, int nseq, int H, 
   // long batches of portions are cut into segments of RT_SEG rows scanned in parallel (two scans and a
   // join instead of one chain of T dependent steps); seg: [T / RT_SEG + nseq][H][Dv][Dk] fp32
   // (max_rows: the longest portion of the batch, known to the host; the grid holds that many segments a sequence)
-  const bool segmented = seg != nullptr && T >= 8 * RT_SEG && max_rows >= 4 * RT_SEG;
+  const bool segmented = seg != nullptr && T >= 8 * RT_SEG && max_rows >= 4 * RT_SEG &&
+                         (max_rows + RT_SEG - 1) / RT_SEG <= RT_JOIN_MAXSEG;
   const int maxseg = (max_rows + RT_SEG - 1) / RT_SEG;
   const long chains = segmented ? (long)T / RT_SEG : nseq;
   // P lanes per group of C value columns (power of two), R rows per lane: P * R >= Dk with R <= 32; a

@@ -83,7 +83,9 @@ CONFIGS = {
                             shared=256, shared_limit=3.0),
                         moe(attn(heads=4, kv=2, dim=64, vdim=32, scale=0.125, far=24, rows=8, kv_from=0, every=9), experts=6, top=2,
                             n=64, limit=3.0, shared=128, shared_limit=3.0),
-                        dense(attn(heads=8, kv=2, dim=32, vdim=64, scale=0.18, far=70, rows=32, coef=0.7, every=33), 256)]},
+                        dense(attn(heads=8, kv=2, dim=32, vdim=64, scale=0.18, far=70, rows=32, coef=0.7, every=33), 256),
+                        # equal key and value widths: decode batches on the split-KV decode kernel
+                        dense(attn(heads=4, kv=1, dim=64, vdim=64, scale=0.125, far=45, rows=12, every=16), 256)]},
 }
 
 

@@ -218,6 +218,43 @@ def test_bucket_edges_and_sinks_on_the_matrix_core_tiles(B, far, hot):
     assert float(got[:, Dv:2 * Dv].abs().max()) < 1e-2          # head 1: swallowed by its sink, towers or not
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D", [(4, 1, 64), (8, 2, 128), (6, 6, 64)])
+def test_split_kv_decode_kernel_takes_bias_and_sink(H, G, D):
+    # the newest row of sequences of 1 .. 700 keys (one partition, several, a merge), as a decode batch
+    dev, B, far, BS = "cuda:0", 14, 90, 16
+    g = torch.Generator().manual_seed(H)
+    lens = [1, 2, 17, 200, 700]
+    relt = rounded(torch.randn(B, H, generator=g), torch.bfloat16)
+    relt[9, 0] = 12.0                                   # distances 29 .. 37 tower for head 0
+    sink = torch.tensor([0.0, 20.0, -30.0, 1.0, 0.5, -0.5, 2.0, 3.0][:H])
+    C = H * D + 2 * G * D
+    nb = sum(-(-n // BS) for n in lens)
+    perm = np.random.default_rng(1).permutation(nb + 2)
+    kc = torch.full((nb + 2, G, BS, D), 50.0, dtype=torch.bfloat16, device=dev)
+    vc = torch.full((nb + 2, G, BS // 8, D, 8), 50.0, dtype=torch.bfloat16, device=dev)
+    eye = torch.eye(C, dtype=F64)
+    W = {"q": eye[:H * D], "k": eye[H * D:H * D + G * D], "v": eye[H * D + G * D:]}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "q_temp": {"coef": 0.3, "every": 64}}
+    bt = np.zeros((len(lens), -(-max(lens) // BS)), dtype=np.int32)
+    qs, want, used = [], [], 0
+    for b, n in enumerate(lens):
+        rows = rounded(torch.randn(n, C, generator=g) * 0.5, torch.bfloat16)
+        k = -(-n // BS)
+        bt[b, :k] = perm[used:used + k]
+        used += k
+        slots = [int(bt[b, t // BS]) * BS + t % BS for t in range(n)]
+        q = ops.qk_norm_pages(rows.to(device=dev, dtype=torch.bfloat16), H, D, G, D, D, i32(np.arange(n), dev), i32(slots, dev),
+                              1e-5, 0.3, 64, kc, vc)
+        qs.append(q[-1])
+        qw, kw_, vw = oracle.attention_qkv(W, "", m, rows.double(), 1e-5)
+        want.append(oracle.attention_core(qw, kw_, vw, relt.double(), sink.double(), 0.05, far)[-1])
+    out = ops.attn_decode(torch.stack(qs).view(len(lens), H, D), kc, vc, i32(bt, dev), i32(lens, dev), 0.05, max(lens),
+                          dist_bias=ops.bucketed_bias(relt, far).to(dev), sink=sink.to(dev))
+    assert rel(out.view(len(lens), -1), torch.stack(want)) < 3e-2
+    assert float(out[:, 1].float().abs().max()) < 1e-2         # head 1: swallowed by its sink
+
+
 # --------------------------------------------------------------------------------------- state-space mixer
 def _mamba_weights(g, H, P, N, G, taps, keep_head0=False):
     C = H * P + 2 * G * N
