@@ -178,7 +178,8 @@ class _Layer:
 class VinozenModel:
     # what this family launches from ops/csrc (ops.require_kernels: a first run compiles only these)
     kernel_sources = ("elementwise.hip", "norm_chain.hip", "rope_pages.hip", "retention.hip", "mamba2.hip",
-                      "attention_mix.hip", "moe_dense.hip", "moe.hip", "sampling.hip", "decode_loop.hip", "gemm_skinny.hip")
+                      "attention_mix.hip", "attention.hip", "moe_dense.hip", "moe.hip", "sampling.hip", "decode_loop.hip",
+                      "gemm_skinny.hip")
     stateful = True         # convolution tails and recurrent state per sequence: state slots, no prefix-cache reuse
     mixed_batches = True    # prompt portions and decode rows of different sequences in one forward
 
