@@ -340,10 +340,22 @@ class VinozenModel:
                 and ops._has("la_attn_decode"))
 
     def prefill_tiles(self, q_lens, device):
-        """(16-row work tiles of the leading prompt portions for ops.attn_mix, rows they cover)."""
+        """((16-row work tiles of the leading prompt portions for ops.attn_mix, 64-row tiles of the same
+        portions for ops.attn_prefill where a layer has the widths that kernel takes), rows they cover)."""
         if device.type != "cuda" or self.f32:
             return None, 0
-        return ops.attn_mix_tiles(q_lens, device)
+        mix, rows = ops.attn_mix_tiles(q_lens, device)
+        pf = None
+        if any(m.kind == "attention" and self._prefill_kernel_ok(m) for m in self.hp.mixers):
+            pf = ops.prefill_tiles(q_lens, device)
+        return (mix, pf), rows
+
+    def _prefill_kernel_ok(self, m: MixSpec) -> bool:
+        """Batches of prompt portions only, for this layer, on the framework's prefill attention kernel (the
+        llama families': 64 query rows of one head per workgroup): bf16, equal key and value widths it is
+        instantiated for; it takes the bias table and the sink."""
+        return (not self.f32 and self.device.type == "cuda" and m.dim == m.vdim and m.dim in (64, 80, 96, 128, 192, 256)
+                and ops._has("la_attn_prefill"))
 
     def _single_rows(self, T: int):
         """(row -> sequence, row ranges, one-row work tiles) of a batch with one row per sequence."""
@@ -427,6 +439,13 @@ class VinozenModel:
             T = q.shape[0]
             return ops.attn_decode(q.view(T, m.heads, m.dim), kv.k[src], kv.v[src], fb.block_tables, fb.seq_lens, m.scale,
                                    fb.max_len, workspace=ws, dist_bias=L.bias, sink=L.sink).view(T, m.heads * m.vdim)
+        if isinstance(tiles, tuple):
+            tiles, pf = tiles
+            if (pf is not None and not fb.decode and tile_rows == q.shape[0] and fb.ctx_lens is not None
+                    and self._prefill_kernel_ok(m) and kv.block_size % 16 == 0):
+                T = q.shape[0]
+                return ops.attn_prefill(q.view(T, m.heads, m.dim), kv.k[src], kv.v[src], cu_q, fb.ctx_lens, fb.block_tables,
+                                        m.scale, tiles=pf, dist_bias=L.bias, sink=L.sink).view(T, m.heads * m.vdim)
         return ops.attn_mix(q, kv.k[src], kv.v[src], row_seq, fb.pos, fb.block_tables, m.heads, m.scale,
                             tiles=tiles, tile_rows=tile_rows, cu_q=cu_q, key_splits=splits, dist_bias=L.bias, sink=L.sink)
 

@@ -88,7 +88,7 @@ def lib():
             "la_dequant": [I, P, P, P, P, I, I, P, P],
             "la_attn_decode": [P, P, P, P, I, P, I, I, I, I, I, F, I, I, P, P, P, P, P, LNG, I, P, P, P, P, F, I, I, P, I, P,
                                P],
-            "la_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, F, P, F, I, P],
+            "la_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, F, P, F, I, P, I, P, P],
             "la_sample": [P, LNG, I, I, P, P, P, P, P],
             "la_penalties": [P, LNG, I, P, I, P, P, I, P, P],
             "la_penalties_cols": [P, LNG, I, P, I, P, P, I, P, I, I, P],
@@ -1667,12 +1667,19 @@ def prefill_tiles(q_lens: Sequence[int], device) -> torch.Tensor:
 def attn_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu_q: torch.Tensor,
                  ctx_lens: torch.Tensor, block_tables: torch.Tensor, scale: float,
                  tiles: Optional[torch.Tensor] = None, q_lens: Optional[Sequence[int]] = None,
-                 out: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0) -> torch.Tensor:
-    """Causal attention for new tokens. q [T,Hq,Dh]; cu_q [nseq+1]; ctx_lens [nseq] (cached+new)."""
+                 out: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0,
+                 dist_bias: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention for new tokens. q [T,Hq,Dh]; cu_q [nseq+1]; ctx_lens [nseq] (cached+new).
+    dist_bias (fp32 [N, Hq]) / sink (fp32 [Hq]): as in attn_decode and attn_mix."""
     T, Hq, Dh = q.shape
     Hkv = k_cache.shape[1]
     if not q.is_cuda:
+        if dist_bias is not None or sink is not None:
+            raise ValueError("attn_prefill: distance bias and sink have no CPU path here (attn_mix has)")
         return _attn_ref_prefill(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, scale, softcap, window)
+    for t in (dist_bias, sink):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda or t.shape[-1] != Hq):
+            raise ValueError("attn_prefill: dist_bias [N, Hq] and sink [Hq] are contiguous fp32")
     if tiles is None:
         cq = cu_q.cpu().tolist()
         tiles = prefill_tiles([cq[i + 1] - cq[i] for i in range(len(cq) - 1)], q.device)
@@ -1681,7 +1688,8 @@ def attn_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     _check(lib().la_attn_prefill(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tiles.data_ptr(),
                                  tiles.shape[0], cu_q.data_ptr(), ctx_lens.data_ptr(), block_tables.data_ptr(),
                                  block_tables.shape[1], Hq, Hkv, Dh, k_cache.shape[2], float(scale),
-                                 out.data_ptr(), float(softcap), int(window), _stream()), "la_attn_prefill")
+                                 out.data_ptr(), float(softcap), int(window), _ptr(dist_bias),
+                                 dist_bias.shape[0] if dist_bias is not None else 0, _ptr(sink), _stream()), "la_attn_prefill")
     return out
 
 

@@ -475,7 +475,8 @@ __global__ __launch_bounds__(PF_T) void attn_prefill_kernel(
     const int* __restrict__ cu_q,           // [nseq+1] token offsets of each seq's queries
     const int* __restrict__ ctx_lens,       // [nseq] total keys (cached + new)
     const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int BS, float scale,
-    bf16* __restrict__ out, float cap, int window, long ldq = 0, long ldk = 0, long ldv = 0, long ldo = 0) {
+    bf16* __restrict__ out, float cap, int window, long ldq = 0, long ldk = 0, long ldv = 0, long ldo = 0,
+    DecExtra E = DecExtra{nullptr, 0, nullptr}) {
   constexpr int DP = (DH + 31) / 32 * 32;  // padded head dim for the MFMA k loop
   constexpr int KC = DP / 32;               // k-chunks of 32
   constexpr int ND = DP / 16;               // 16-wide output column tiles
@@ -513,7 +514,10 @@ __global__ __launch_bounds__(PF_T) void attn_prefill_kernel(
   for (int i = 0; i < ND; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float mrow[4], lrow[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { mrow[i] = -INFINITY; lrow[i] = 0.f; }
+  for (int i = 0; i < 4; ++i) {   // a sink: the softmax state starts at (sink, 1) instead of (-inf, 0)
+    mrow[i] = E.sink ? E.sink[h] * 1.4426950408889634f : -INFINITY;
+    lrow[i] = E.sink ? 1.f : 0.f;
+  }
 
   const float sl2 = scale * 1.4426950408889634f;
   const int last_row = min(qlen, r0 + 64) - 1;
@@ -588,6 +592,10 @@ __global__ __launch_bounds__(PF_T) void attn_prefill_kernel(
         v1 = cap * 1.4426950408889634f * tanhf(sacc[1][i] * scale / cap);
       }
       const int key0 = k0 + fr, key1 = k0 + 16 + fr;
+      if (E.bias) {   // bias per distance and head, constant from the table's last row on
+        v0 = fmaf(E.bias[(long)min(max(qpos - key0, 0), E.nbias - 1) * Hq + h], 1.4426950408889634f, v0);
+        v1 = fmaf(E.bias[(long)min(max(qpos - key1, 0), E.nbias - 1) * Hq + h], 1.4426950408889634f, v1);
+      }
       const int wlo = window > 0 ? qpos - window + 1 : 0;
       const bool causal = !DENSE;
       if ((causal && key0 > qpos) || key0 >= kend || qr >= qlen || key0 < wlo) v0 = -INFINITY;
@@ -744,14 +752,15 @@ extern "C" int la_attn_dense(const void* q, long ldq, const void* k, long ldk, c
 extern "C" int la_attn_prefill(const void* q, const void* kc, const void* vc, const int* tiles, int ntiles,
                                const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks, int Hq,
                                int Hkv, int Dh, int BS, float scale, void* out, float softcap, int window,
-                               void* stream) {
-  if (Hq % Hkv) return -1;
+                               const float* dist_bias, int nbias, const float* sink, void* stream) {
+  if (Hq % Hkv || (dist_bias && nbias < 1)) return -1;
+  const la::DecExtra E{dist_bias, nbias, sink};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(ntiles, Hq);
 #define PF(D)                                                                                                     \
   hipLaunchKernelGGL(la::attn_prefill_kernel<D>, grid, dim3(la::PF_T), 0, st, (const bf16*)q, (const bf16*)kc,    \
                      (const bf16*)vc, tiles, cu_q, ctx_lens, block_tables, max_blocks, Hq, Hkv, BS, scale,       \
-                     (bf16*)out, softcap, window)
+                     (bf16*)out, softcap, window, 0L, 0L, 0L, 0L, E)
   switch (Dh) {
     case 64: PF(64); break;
     case 80: PF(80); break;

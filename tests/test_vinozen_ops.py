@@ -255,6 +255,45 @@ def test_split_kv_decode_kernel_takes_bias_and_sink(H, G, D):
     assert float(out[:, 1].float().abs().max()) < 1e-2         # head 1: swallowed by its sink
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D", [(4, 1, 64), (4, 2, 128)])
+def test_prefill_kernel_takes_bias_and_sink(H, G, D):
+    # a batch of three portions: one continuing after 50 cached rows, one from position 0, one of a single row
+    dev, B, far, BS = "cuda:0", 14, 90, 16
+    g = torch.Generator().manual_seed(H + D)
+    relt = rounded(torch.randn(B, H, generator=g), torch.bfloat16)
+    relt[9, 0] = 12.0
+    sink = torch.tensor([0.0, 20.0, -30.0, 1.0])
+    C = H * D + 2 * G * D
+    spans = [(50, 150), (0, 37), (20, 21)]              # (first row of the portion, end) per sequence
+    nb = sum(-(-e // BS) for _, e in spans)
+    perm = np.random.default_rng(2).permutation(nb + 2)
+    kc = torch.full((nb + 2, G, BS, D), 50.0, dtype=torch.bfloat16, device=dev)
+    vc = torch.full((nb + 2, G, BS // 8, D, 8), 50.0, dtype=torch.bfloat16, device=dev)
+    eye = torch.eye(C, dtype=F64)
+    W = {"q": eye[:H * D], "k": eye[H * D:H * D + G * D], "v": eye[H * D + G * D:]}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "q_temp": {"coef": 0.3, "every": 64}}
+    bt = np.zeros((len(spans), -(-max(e for _, e in spans) // BS)), dtype=np.int32)
+    qs, want, used = [], [], 0
+    for b, (a, e) in enumerate(spans):
+        rows = rounded(torch.randn(e, C, generator=g) * 0.5, torch.bfloat16)
+        k = -(-e // BS)
+        bt[b, :k] = perm[used:used + k]
+        used += k
+        slots = [int(bt[b, t // BS]) * BS + t % BS for t in range(e)]
+        q = ops.qk_norm_pages(rows.to(device=dev, dtype=torch.bfloat16), H, D, G, D, D, i32(np.arange(e), dev), i32(slots, dev),
+                              1e-5, 0.3, 64, kc, vc)
+        qs.append(q[a:])
+        qw, kw_, vw = oracle.attention_qkv(W, "", m, rows.double(), 1e-5)
+        want.append(oracle.attention_core(qw, kw_, vw, relt.double(), sink.double(), 0.05, far)[a:])
+    qlens = [e - a for a, e in spans]
+    out = ops.attn_prefill(torch.cat(qs).view(-1, H, D), kc, vc, i32(np.cumsum([0] + qlens), dev), i32([e for _, e in spans], dev),
+                           i32(bt, dev), 0.05, tiles=ops.prefill_tiles(qlens, dev),
+                           dist_bias=ops.bucketed_bias(relt, far).to(dev), sink=sink.to(dev))
+    assert rel(out.view(sum(qlens), -1), torch.cat(want)) < 3e-2
+    assert float(out[:, 1].float().abs().max()) < 1e-2         # head 1: swallowed by its sink
+
+
 # --------------------------------------------------------------------------------------- state-space mixer
 def _mamba_weights(g, H, P, N, G, taps, keep_head0=False):
     C = H * P + 2 * G * N
