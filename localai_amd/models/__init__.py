@@ -9,7 +9,8 @@ import importlib
 # architecture -> (module, class); imported lazily: some families pull in optional dependencies
 MODEL_CLASSES = {"suganex": ("localai_amd.models.suganex", "SuganexModel"),
                  "dadizen": ("localai_amd.models.dadizen", "DadizenModel"),
-                 "vinozen": ("localai_amd.models.vinozen", "VinozenModel")}
+                 "vinozen": ("localai_amd.models.vinozen", "VinozenModel"),
+                 "gosuvik": ("localai_amd.models.gosuvik", "GosuvikModel")}
 
 
 def model_class(arch: str):

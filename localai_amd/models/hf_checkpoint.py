@@ -65,7 +65,7 @@ QUANT_MODES = {"bnb_4bit": "q4_k_m", "xpu_4bit": "q4_k_m", "q4_k_m": "q4_k_m", "
 
 # checkpoint directories whose config.json names ONE design under "architecture" and lists its
 # layers one by one ("layers": [{type, mixer, mlp}, ...]): design name -> engine architecture
-LAYERED_ARCH_OF = {"Suganex": "suganex", "Dadizen": "dadizen", "Vinozen": "vinozen"}
+LAYERED_ARCH_OF = {"Suganex": "suganex", "Dadizen": "dadizen", "Vinozen": "vinozen", "Gosuvik": "gosuvik"}
 
 
 def layered_architecture(path: str) -> str:

@@ -133,6 +133,15 @@ def lib():
                           P],
             "la_attn_latent": [P, P, P, P, P, I, I, I, I, I, I, F, I, P, I, P, I, P, P, P],
             "la_norm_chain": [P, I, I, P, I, LNG, I, I, F, P, P, F, P, I, I, F, P, P, P, I, P],
+            "la_add_group_norm": [P, I, I, P, I, LNG, I, P, F, I, P, I, P],
+            "la_poly_norm_act": [P, I, LNG, I, I, I, P, F, P, I, P],
+            "la_sigmoid_mul": [P, I, P, I, LNG, I, I, P, I, P],
+            "la_qk_norm_rope_pages": [I, P, LNG, I, I, I, I, I, P, P, P, P, F, P, F, I, P, P, P, P, I, P],
+            "la_rotate_heads": [I, P, I, I, I, P, P, F, F, P, LNG, P],
+            "la_delta_rule": [I, P, LNG, P, P, I, I, I, I, I, I, I, I, P, P, P, P, F, F, P, P, P, P, P, I, P, P, P, P, P,
+                              P, P],
+            "la_matrix_memory": [I, P, LNG, I, I, I, I, I, P, F, P, F, F, F, P, P, P, P, P, I, P, P, P, P, P, LNG, P, I,
+                                 P],
             "la_glu_clamp": [P, I, LNG, I, I, I, F, F, P, I, P],
             "la_side_gate": [P, I, LNG, I, I, I, P, P, I, I, P, I, P],
             "la_rope_pages": [I, P, I, I, I, I, I, I, P, P, P, F, I, I, I, P, P, P, I, P],
@@ -2600,6 +2609,370 @@ def mamba2(src: torch.Tensor, H: int, P: int, N: int, G: int, conv_w: torch.Tens
                            int(norm_groups), float(eps), pos.data_ptr(), cu_q.data_ptr(), sslots.data_ptr(),
                            conv_state.data_ptr(), ssm_state.data_ptr(), int(T == nseq and max_rows == 1), xs.data_ptr(), cb.data_ptr(),
                            dtd.data_ptr(), o.data_ptr(), out.data_ptr(), _ptr(seg), max_rows, _stream()), "la_mamba2")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# Layer-list designs: grouped input norms, polynomial activations, normed rotated pages with
+# rotated values, the gated delta rule with a decay per key channel, stabilised matrix memories
+# ---------------------------------------------------------------------------------------
+
+def _group_rms_ref(x: torch.Tensor, w: torch.Tensor, eps: float, groups: int) -> torch.Tensor:
+    T, D = x.shape
+    g = x.reshape(T, groups, D // groups)
+    return (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, D) * w.float()
+
+
+def add_group_norm(res: torch.Tensor, branch, w: torch.Tensor, eps: float, groups: int = 1,
+                   out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Sublayer boundary of a pre-normed fp32 residual stream (fp32 [T, D], updated in place):
+    res <- res + branch (a Partial or dense [T, D] tensor; None: the stream is only read), then
+    returns the stream normed in `groups` equal consecutive parts, each divided by its own
+    sqrt(mean(part^2) + eps), the whole times w (fp32 [D]).  All arithmetic fp32."""
+    T, D = res.shape
+    if groups < 1 or D % groups or w.numel() != D:
+        raise ValueError("add_group_norm: the width is a multiple of the group count, w is [D]")
+    if not res.is_cuda:
+        if branch is not None:
+            res += _branch_dense(branch)
+        return _group_rms_ref(res, w, eps, groups).to(out_dtype)
+    if res.dtype != torch.float32 or not res.is_contiguous() or out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("add_group_norm: the stream is contiguous fp32; outputs are bf16 or fp32")
+    if w.dtype != torch.float32 or not w.is_contiguous():
+        raise ValueError("add_group_norm: weights are contiguous fp32 [D]")
+    a = _branch_args(branch, T, D) if branch is not None else (None, 0, 0, 0)
+    out = torch.empty(T, D, dtype=out_dtype, device=res.device)
+    _check(lib().la_add_group_norm(res.data_ptr(), T, D, a[0], a[1], a[2], a[3], w.data_ptr(), float(eps), int(groups),
+                                   out.data_ptr(), int(out_dtype == torch.float32), _stream()), "la_add_group_norm")
+    return out
+
+
+def poly_norm_act(src, coef: torch.Tensor, eps: float, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Polynomial activation with unit powers on a projection z [T, F]:  y = a N(z) + b N(z^2) + c
+    N(z^3) + e, powers element by element, N(u) = u / sqrt(mean_F(u^2) + eps) over the row, (a, b,
+    c, e) = coef (fp32 [4], on z's device).  fp32 arithmetic, [T, F] in out_dtype."""
+    t = src.t if isinstance(src, Partial) else src
+    T, F = t.shape[-2], t.shape[-1]
+    if coef.numel() != 4:
+        raise ValueError("poly_norm_act: four coefficients")
+    if not t.is_cuda:
+        z = _branch_dense(src)
+        cf = coef.float()
+        n = lambda u: u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)  # noqa: E731
+        return (cf[0] * n(z) + cf[1] * n(z * z) + cf[2] * n(z * z * z) + cf[3]).to(out_dtype)
+    if coef.dtype != torch.float32 or not coef.is_cuda:
+        raise ValueError("poly_norm_act: coefficients are fp32 on the device")
+    a = _branch_args(src, T, F)
+    out = torch.empty(T, F, dtype=out_dtype, device=t.device)
+    _check(lib().la_poly_norm_act(a[0], a[1], a[2], a[3], T, F, coef.data_ptr(), float(eps), out.data_ptr(),
+                                  int(out_dtype == torch.float32), _stream()), "la_poly_norm_act")
+    return out
+
+
+def sigmoid_mul(x: torch.Tensor, gate: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x * sigmoid(gate), element by element: x [T, N] contiguous, gate a [T, N] view with unit
+    column stride (the gate columns of a wider projection); fp32 arithmetic."""
+    T, N = x.shape
+    out_dtype = out_dtype or x.dtype
+    if tuple(gate.shape) != (T, N) or gate.stride(1) != 1:
+        raise ValueError("sigmoid_mul: the gate is a [T, N] view with unit column stride")
+    if not x.is_cuda:
+        return (x.float() * torch.sigmoid(gate.float())).to(out_dtype)
+    if (x.dtype not in (torch.float32, torch.bfloat16) or gate.dtype not in (torch.float32, torch.bfloat16)
+            or not x.is_contiguous() or out_dtype not in (torch.float32, torch.bfloat16)):
+        raise ValueError("sigmoid_mul: bf16 or fp32 operands, x contiguous")
+    out = torch.empty(T, N, dtype=out_dtype, device=x.device)
+    _check(lib().la_sigmoid_mul(x.data_ptr(), int(x.dtype == torch.float32), gate.data_ptr(),
+                                int(gate.dtype == torch.float32), gate.stride(0), T, N, out.data_ptr(),
+                                int(out_dtype == torch.float32), _stream()), "la_sigmoid_mul")
+    return out
+
+
+def linear_rot_freqs(dims: int, base: float, factor: float = 1.0, device=None) -> torch.Tensor:
+    """Angular frequencies fp32 [dims / 2] of a rotation whose positions are divided by `factor`
+    (linear position scaling): f_i = base^(-2i / dims) / factor; float64 on the host."""
+    f = np.power(float(base), -2.0 * np.arange(dims // 2, dtype=np.float64) / dims) / float(factor)
+    return torch.from_numpy(f.astype(np.float32)).to(device)
+
+
+def qk_norm_rope_pages(src: torch.Tensor, H: int, D: int, G: int, Dv: int, pos: torch.Tensor, slots: torch.Tensor,
+                       q_w: torch.Tensor, k_w: torch.Tensor, eps: float, freqs: torch.Tensor, mag: float, rot: int,
+                       v_freqs: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+    """Normed, rotated queries and keys and rotated values: of projection rows src [T, >= H D + G D
+    + G Dv] (q | k | v, any row stride) every query and key head is divided by sqrt(mean x^2 + eps)
+    and multiplied by q_w / k_w (fp32 [D], shared by the heads); then dims i and i + rot / 2 of its
+    first `rot` dims are turned by the angle pos * freqs[i] (cos, sin times mag).  With v_freqs
+    (fp32 [Dv / 2]) every value head is turned the same way over its whole width, dims m and m + Dv
+    / 2 by pos * v_freqs[m], so that the cache holds values in the frame of their own position (an
+    attention output is turned back by its query's position: rotate_heads).  Returns q [T, H D];
+    keys and values go to the paged pools (K [blocks, G, BS, D], V [blocks, G, BS / 8, Dv, 8]) at
+    `slots` (-1: nowhere).  Norms, angles and rotations fp32."""
+    T = src.shape[0]
+    Cq, Ck, Cv = H * D, G * D, G * Dv
+    if (src.dim() != 2 or src.shape[1] < Cq + Ck + Cv or pos.shape[0] != T or src.stride(1) != 1 or rot % 2 or rot > D
+            or freqs.numel() != rot // 2 or q_w.numel() != D or k_w.numel() != D or slots.shape[0] != T
+            or (v_freqs is not None and (Dv % 2 or v_freqs.numel() != Dv // 2))):
+        raise ValueError("qk_norm_rope_pages: operand shapes do not fit")
+    if (tuple(k_cache.shape[1:]) != (G, k_cache.shape[2], D)
+            or tuple(v_cache.shape[1:]) != (G, k_cache.shape[2] // 8, Dv, 8)):
+        raise ValueError("qk_norm_rope_pages: pools do not fit the key / value widths")
+    if not src.is_cuda:
+        x = src.float()
+        nrm = lambda y, w: y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
+        q = _rotate_ref(nrm(x[:, :Cq].reshape(T, H, D), q_w), pos, freqs, mag, rot, 0, False)
+        k = _rotate_ref(nrm(x[:, Cq:Cq + Ck].reshape(T, G, D), k_w), pos, freqs, mag, rot, 0, False)
+        v = x[:, Cq + Ck:Cq + Ck + Cv].reshape(T, G, Dv)
+        if v_freqs is not None:
+            v = _rotate_ref(v, pos, v_freqs, 1.0, Dv, 0, False)
+        _page_write_ref(k_cache, v_cache, slots, k, v)
+        return q.reshape(T, Cq).to(src.dtype)
+    if src.dtype not in (torch.float32, torch.bfloat16) or k_cache.dtype != src.dtype or v_cache.dtype != src.dtype:
+        raise ValueError("qk_norm_rope_pages: bf16 or fp32 rows, pools of the same dtype")
+    assert pos.dtype == torch.int32 and slots.dtype == torch.int32
+    for t in (q_w, k_w, freqs, v_freqs):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda)
+    q = torch.empty(T, Cq, dtype=src.dtype, device=src.device)
+    _check(lib().la_qk_norm_rope_pages(int(src.dtype == torch.float32), src.data_ptr(), src.stride(0), T, H, D, G, Dv,
+                                       pos.data_ptr(), slots.data_ptr(), q_w.data_ptr(), k_w.data_ptr(), float(eps),
+                                       freqs.data_ptr(), float(mag), rot, _ptr(v_freqs), q.data_ptr(), k_cache.data_ptr(),
+                                       v_cache.data_ptr(), k_cache.shape[2], _stream()), "la_qk_norm_rope_pages")
+    return q
+
+
+def rotate_heads(x: torch.Tensor, H: int, Dv: int, pos: torch.Tensor, freqs: torch.Tensor, sign: float = -1.0,
+                 scale: float = 1.0, out: Optional[torch.Tensor] = None, col0: int = 0) -> torch.Tensor:
+    """Every head of x [T, H Dv] turned over its whole width, dims m and m + Dv / 2 by the angle
+    sign * pos * freqs[m] (fp32), times `scale`; written to out[:, col0 : col0 + H Dv] (a new [T, H
+    Dv] tensor of x's dtype when out is None).  sign -1 takes an attention output over values
+    cached in the frame of their own positions back to the frame of its query."""
+    T = x.shape[0]
+    N = H * Dv
+    if x.dim() != 2 or x.shape[1] != N or Dv % 2 or freqs.numel() != Dv // 2 or pos.shape[0] != T:
+        raise ValueError("rotate_heads: operand shapes do not fit")
+    if out is None:
+        out, col0 = torch.empty(T, N, dtype=x.dtype, device=x.device), 0
+    if out.shape[0] != T or col0 < 0 or col0 + N > out.shape[1] or out.stride(1) != 1 or out.dtype != x.dtype:
+        raise ValueError("rotate_heads: the output window does not fit")
+    if not x.is_cuda:
+        y = _rotate_ref(x.float().reshape(T, H, Dv), pos.float() * sign, freqs, 1.0, Dv, 0, False) * scale
+        out[:, col0:col0 + N] = y.reshape(T, N).to(out.dtype)
+        return out
+    if x.dtype not in (torch.float32, torch.bfloat16) or not x.is_contiguous():
+        raise ValueError("rotate_heads: contiguous bf16 or fp32 rows")
+    assert pos.dtype == torch.int32 and freqs.dtype == torch.float32 and freqs.is_contiguous()
+    es = x.element_size()
+    _check(lib().la_rotate_heads(int(x.dtype == torch.float32), x.data_ptr(), T, H, Dv, pos.data_ptr(), freqs.data_ptr(),
+                                 float(sign), float(scale), out.data_ptr() + col0 * es, out.stride(0), _stream()),
+           "la_rotate_heads")
+    return out
+
+
+def _conv_hist_ref(state, ss, p0, taps, C):
+    """The taps - 1 rows before a portion that starts at position p0: the slot's tail, zeros before position 0."""
+    hist = torch.zeros(max(taps - 1, 0), C)
+    if taps > 1:
+        hist = state[ss].float().clone()
+        for i in range(taps - 1):            # state row i holds position p0 - (taps - 1) + i
+            if p0 - (taps - 1) + i < 0:
+                hist[i] = 0
+    return hist
+
+
+def delta_rule_states(slots: int, H: int, G: int, Dk: int, Dv: int, taps: int, dtype=torch.bfloat16, device=None):
+    """State pools of ops.delta_rule: (convolution tails [slots, taps - 1, 2 G Dk + H Dv] of the
+    activation dtype, recurrent state fp32 [slots, H, Dv, Dk], value-column major)."""
+    return (torch.zeros(slots, max(taps - 1, 0), 2 * G * Dk + H * Dv, dtype=dtype, device=device),
+            torch.zeros(slots, H, Dv, Dk, dtype=torch.float32, device=device))
+
+
+def delta_rule(src: torch.Tensor, dec: torch.Tensor, gate: torch.Tensor, H: int, G: int, Dk: int, Dv: int,
+               conv_w: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, norm_w: torch.Tensor, eps: float,
+               pos: torch.Tensor, cu_q: torch.Tensor, sslots: torch.Tensor, conv_state: torch.Tensor,
+               rec_state: torch.Tensor, unit_eps: float = 1e-6, max_rows: int = 0) -> torch.Tensor:
+    """Gated delta rule with one decay per head and key channel over projection rows src [T, >= 2 G
+    Dk + H Dv + H] laid out [q | k | v | beta logits] (any row stride), dec [T, H Dk] (decay
+    logits) and gate [T, H Dv] (output gate logits):
+      * q, k (G heads of width Dk; head h reads group floor(h / (H / G))) and v (H heads of width
+        Dv) pass a depthwise causal convolution over time (conv_w [2 G Dk + H Dv, taps] fp32, last
+        tap = current token, no bias, zeros before position 0) and silu;
+      * q and k become unit vectors per head, x / sqrt(sum x^2 + unit_eps); q times Dk^-1/2;
+      * beta = sigmoid(beta logits); g = exp(-exp(a_log[h]) softplus(dec + dt_bias)) per (head, key channel);
+      * per head, S (Dk x Dv):  S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q;
+      * o divided by its root mean square over the head's Dv (eps), times norm_w (fp32 [Dv], shared
+        by the heads), times sigmoid(gate).
+    Rows of a sequence portion are consecutive (cu_q [nseq + 1], pos [T]); the portion's history
+    comes from conv_state[sslots[seq]] (the last taps - 1 rows of [q | k | v] before the
+    convolution) and rec_state[sslots[seq]] (fp32 [H, Dv, Dk]), both taken as zero before position
+    0, and both are advanced to the portion's end.  Everything after the convolution's silu is
+    fp32.  Returns [T, H Dv] in src's dtype."""
+    T = src.shape[0]
+    nseq = cu_q.shape[0] - 1
+    Cqk, Cv = G * Dk, H * Dv
+    C = 2 * Cqk + Cv
+    taps = conv_w.shape[1]
+    if (src.dim() != 2 or src.shape[1] < C + H or src.stride(1) != 1 or H % G or conv_w.shape[0] != C
+            or tuple(dec.shape) != (T, H * Dk) or tuple(gate.shape) != (T, Cv)
+            or tuple(conv_state.shape[1:]) != (max(taps - 1, 0), C) or tuple(rec_state.shape[1:]) != (H, Dv, Dk)
+            or dt_bias.numel() != H * Dk or a_log.numel() != H or norm_w.numel() != Dv or sslots.shape[0] != nseq
+            or pos.shape[0] != T):
+        raise ValueError("delta_rule: operand shapes do not fit")
+    if not src.is_cuda:
+        u_ = src[:, :C].float()
+        beta = torch.sigmoid(src[:, C:C + H].float())
+        dt = torch.nn.functional.softplus(dec.float() + dt_bias.float(), threshold=1e9).view(T, H, Dk)
+        gdec = torch.exp(-torch.exp(a_log.float()).view(1, H, 1) * dt)
+        o = torch.zeros(T, H, Dv)
+        cu = cu_q.tolist()
+        rep = H // G
+        for s in range(nseq):
+            a, b = cu[s], cu[s + 1]
+            if b <= a:
+                continue
+            ss, p0 = int(sslots[s]), int(pos[a])
+            ext = torch.cat([_conv_hist_ref(conv_state, ss, p0, taps, C), u_[a:b]], 0)
+            c = torch.zeros(b - a, C)
+            for j in range(taps):
+                c = c + conv_w[:, j].float() * ext[j:j + (b - a)]
+            c = torch.nn.functional.silu(c)
+            if taps > 1:
+                conv_state[ss] = ext[-(taps - 1):].to(conv_state.dtype)
+            q = c[:, :Cqk].reshape(-1, G, Dk)
+            k = c[:, Cqk:2 * Cqk].reshape(-1, G, Dk)
+            q = (q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + unit_eps) * Dk ** -0.5).repeat_interleave(rep, 1)
+            k = (k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, 1)
+            v = c[:, 2 * Cqk:].reshape(-1, H, Dv)
+            S = torch.zeros(H, Dk, Dv) if p0 == 0 else rec_state[ss].float().transpose(1, 2).clone()
+            for t in range(b - a):
+                S = gdec[a + t].unsqueeze(2) * S
+                uu = beta[a + t].view(H, 1) * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
+                S = S + k[t].unsqueeze(2) * uu.unsqueeze(1)
+                o[a + t] = torch.einsum("hkv,hk->hv", S, q[t])
+            rec_state[ss] = S.transpose(1, 2)
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+        return (o.reshape(T, Cv) * torch.sigmoid(gate.float())).to(src.dtype)
+    f32 = src.dtype == torch.float32
+    if src.dtype not in (torch.float32, torch.bfloat16) or conv_state.dtype != src.dtype or dec.dtype != src.dtype \
+            or gate.dtype != src.dtype or not dec.is_contiguous() or not gate.is_contiguous():
+        raise ValueError("delta_rule: bf16 or fp32 rows; tails, decay and gate logits of the same dtype")
+    if rec_state.dtype != torch.float32 or not rec_state.is_contiguous() or not conv_state.is_contiguous():
+        raise ValueError("delta_rule: the recurrent state pool is contiguous fp32")
+    for t in (pos, cu_q, sslots):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    for t in (conv_w, dt_bias, a_log, norm_w):
+        assert t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda
+    dev = src.device
+    qk = torch.empty(T, 2 * Cqk, dtype=torch.float32, device=dev)       # unit q (scaled) | unit k per group
+    vf = torch.empty(T, Cv, dtype=torch.float32, device=dev)            # convolved v
+    gd = torch.empty(T, H * Dk, dtype=torch.float32, device=dev)        # decays per (token, head, key channel)
+    bq = torch.empty(T, H + G, dtype=torch.float32, device=dev)         # beta per head | k . q per group
+    o = torch.empty(T, Cv, dtype=torch.float32, device=dev)
+    out = torch.empty(T, Cv, dtype=src.dtype, device=dev)
+    max_rows = int(max_rows) if max_rows > 0 else T
+    _check(lib().la_delta_rule(int(f32), src.data_ptr(), src.stride(0), dec.data_ptr(), gate.data_ptr(), T, nseq, H, G, Dk,
+                               Dv, taps, rec_state.shape[0], conv_w.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(),
+                               norm_w.data_ptr(), float(eps), float(unit_eps), pos.data_ptr(), cu_q.data_ptr(),
+                               sslots.data_ptr(), conv_state.data_ptr(), rec_state.data_ptr(),
+                               int(T == nseq and max_rows == 1), qk.data_ptr(), vf.data_ptr(), gd.data_ptr(), bq.data_ptr(),
+                               o.data_ptr(), out.data_ptr(), _stream()), "la_delta_rule")
+    return out
+
+
+def matrix_memory_states(slots: int, H: int, Dk: int, Dv: int, device=None):
+    """State pools of ops.matrix_memory: (fp32 [slots, H, Dv + 1, Dk]: the Dk x Dv memory
+    value-column major with the normaliser vector as one more column, fp32 [slots, H]: the running
+    maximum of the gates' logarithms)."""
+    return (torch.zeros(slots, H, Dv + 1, Dk, dtype=torch.float32, device=device),
+            torch.zeros(slots, H, dtype=torch.float32, device=device))
+
+
+def matrix_memory(src: torch.Tensor, H: int, Dk: int, Dv: int, gate_b: torch.Tensor, cap: float, norm_w: torch.Tensor,
+                  eps: float, pos: torch.Tensor, cu_q: torch.Tensor, sslots: torch.Tensor, mem_state: torch.Tensor,
+                  max_state: torch.Tensor, scale: float = 1.0, denom_eps: float = 1e-6, max_rows: int = 0,
+                  out: Optional[torch.Tensor] = None, col0: int = 0) -> torch.Tensor:
+    """Matrix memory with exponential gates kept in range by a running maximum, over projection
+    rows src [T, >= 2 H Dk + 2 H Dv + 2 H] laid out [q | k | v | output gate | input gate | forget
+    gate] (any row stride); gate_b fp32 [2 H]: the input and forget gates' biases.  Per head:
+      i = cap tanh((input + b) / cap),  f = logsigmoid(cap tanh((forget + b) / cap)),  q times Dk^-1/2;
+      m' = max(f + m, i);  S <- exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k alone;
+      o = S^T q / (max(|n . q|, exp(-m')) + denom_eps);
+    o divided by its root mean square over the head's Dv (eps), times norm_w (fp32 [H Dv]), times
+    sigmoid(output gate), times `scale`.  S, n and m of a sequence live in mem_state[sslots[seq]]
+    (fp32 [H, Dv + 1, Dk], n as the last column) and max_state[sslots[seq]] (fp32 [H]); all start at
+    zero at position 0 (m too) and are advanced to the portion's end.  Gates, the recurrence and the
+    norm are fp32.  Written to out[:, col0 : col0 + H Dv] (a new tensor of src's dtype when None)."""
+    T = src.shape[0]
+    nseq = cu_q.shape[0] - 1
+    Cq, Cv = H * Dk, H * Dv
+    W = 2 * Cq + 2 * Cv + 2 * H
+    if (src.dim() != 2 or src.shape[1] < W or src.stride(1) != 1 or tuple(mem_state.shape[1:]) != (H, Dv + 1, Dk)
+            or tuple(max_state.shape[1:]) != (H,) or gate_b.numel() != 2 * H or norm_w.numel() != Cv
+            or sslots.shape[0] != nseq or pos.shape[0] != T):
+        raise ValueError("matrix_memory: operand shapes do not fit")
+    if out is None:
+        out, col0 = torch.empty(T, Cv, dtype=src.dtype, device=src.device), 0
+    if out.shape[0] != T or col0 < 0 or col0 + Cv > out.shape[1] or out.stride(1) != 1 or out.dtype != src.dtype:
+        raise ValueError("matrix_memory: the output window does not fit")
+    if not src.is_cuda:
+        x = src.float()
+        q = x[:, :Cq].reshape(T, H, Dk) * Dk ** -0.5
+        k = x[:, Cq:2 * Cq].reshape(T, H, Dk)
+        v = x[:, 2 * Cq:2 * Cq + Cv].reshape(T, H, Dv)
+        og = x[:, 2 * Cq + Cv:2 * Cq + 2 * Cv]
+        b = gate_b.float()
+        ig = cap * torch.tanh((x[:, W - 2 * H:W - H] + b[:H]) / cap)
+        fg = torch.nn.functional.logsigmoid(cap * torch.tanh((x[:, W - H:W] + b[H:]) / cap))
+        o = torch.zeros(T, H, Dv)
+        cu = cu_q.tolist()
+        for s in range(nseq):
+            a, e = cu[s], cu[s + 1]
+            if e <= a:
+                continue
+            ss = int(sslots[s])
+            if int(pos[a]) == 0:
+                S, n, m = torch.zeros(H, Dk, Dv), torch.zeros(H, Dk), torch.zeros(H)
+            else:
+                st = mem_state[ss].float()
+                S, n, m = st[:, :Dv].transpose(1, 2).clone(), st[:, Dv].clone(), max_state[ss].float().clone()
+            for t in range(a, e):
+                m2 = torch.maximum(fg[t] + m, ig[t])
+                fa, ia = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
+                S = fa.view(H, 1, 1) * S + ia.view(H, 1, 1) * k[t].unsqueeze(2) * v[t].unsqueeze(1)
+                n = fa.view(H, 1) * n + ia.view(H, 1) * k[t]
+                m = m2
+                den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + denom_eps
+                o[t] = torch.einsum("hkv,hk->hv", S, q[t]) / den.view(H, 1)
+            mem_state[ss, :, :Dv] = S.transpose(1, 2)
+            mem_state[ss, :, Dv] = n
+            max_state[ss] = m
+        o = (o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, Cv)
+        out[:, col0:col0 + Cv] = (o * norm_w.float() * torch.sigmoid(og) * scale).to(out.dtype)
+        return out
+    f32 = src.dtype == torch.float32
+    if src.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("matrix_memory: bf16 or fp32 rows")
+    if (mem_state.dtype != torch.float32 or max_state.dtype != torch.float32 or not mem_state.is_contiguous()
+            or not max_state.is_contiguous()):
+        raise ValueError("matrix_memory: the state pools are contiguous fp32")
+    for t in (pos, cu_q, sslots):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    for t in (gate_b, norm_w):
+        assert t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda
+    dev = src.device
+    Dv1 = Dv + 1
+    qk = torch.empty(T, 2 * Cq, dtype=torch.float32, device=dev)       # scaled q | k
+    va = torch.empty(T, H * Dv1, dtype=torch.float32, device=dev)      # v with a column of ones per head
+    gts = torch.empty(T, 3 * H, dtype=torch.float32, device=dev)       # decay | input scale | exp(-m) per (token, head)
+    o = torch.empty(T, H * Dv1, dtype=torch.float32, device=dev)
+    max_rows = int(max_rows) if max_rows > 0 else T
+    seg = torch.empty((T // RETENTION_SEG + nseq) * H * Dv1 * Dk, dtype=torch.float32, device=dev) \
+        if (T >= 8 * RETENTION_SEG and max_rows >= 4 * RETENTION_SEG) else None
+    es = src.element_size()
+    _check(lib().la_matrix_memory(int(f32), src.data_ptr(), src.stride(0), T, nseq, H, Dk, Dv, gate_b.data_ptr(), float(cap),
+                                  norm_w.data_ptr(), float(eps), float(denom_eps), float(scale), pos.data_ptr(),
+                                  cu_q.data_ptr(), sslots.data_ptr(), mem_state.data_ptr(), max_state.data_ptr(),
+                                  mem_state.shape[0], qk.data_ptr(), va.data_ptr(), gts.data_ptr(), o.data_ptr(),
+                                  out.data_ptr() + col0 * es, out.stride(0), _ptr(seg), max_rows, _stream()),
+           "la_matrix_memory")
     return out
 
 
