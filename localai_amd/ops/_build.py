@@ -31,7 +31,8 @@ def _torch_lib() -> str:
 _NO_PK_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]   # scalar fp32 math only
 FILE_FLAGS = {"gemm_bs.hip": ["-fno-slp-vectorize"], "shortconv.hip": _NO_PK_F32, "attention_mix.hip": _NO_PK_F32,
               "moe_dense.hip": _NO_PK_F32, "norm_chain.hip": _NO_PK_F32, "rope_pages.hip": _NO_PK_F32,
-              "retention.hip": _NO_PK_F32, "attention_latent.hip": _NO_PK_F32, "mamba2.hip": _NO_PK_F32}
+              "retention.hip": _NO_PK_F32, "attention_latent.hip": _NO_PK_F32, "mamba2.hip": _NO_PK_F32, "delta_rule.hip": _NO_PK_F32,
+              "matrix_memory.hip": _NO_PK_F32}
 
 
 def _sources():

@@ -1,0 +1,344 @@
+// Gated delta rule with one decay per head and key channel.
+//
+//   [q | k | v] rows pass a depthwise causal convolution over time and silu;  q, k (G heads of width Dk,
+//   head h reads group h / (H / G)) become unit vectors, x / sqrt(sum x^2 + unit_eps), q times Dk^-1/2;
+//   beta_h = sigmoid(.);  g_(h,d) = exp(-exp(a_log_h) softplus(dec_(h,d) + dt_bias_(h,d)));  per head, S (Dk x Dv):
+//       S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+//   out = o / sqrt(mean_d o^2 + eps) * w_d * sigmoid(gate)                      (mean over the head's Dv)
+//
+// Per-sequence state between launches: the last taps - 1 rows of [q | k | v] before the convolution
+// ([slots][taps - 1][C], the activation type) and S ([slots][H][Dv][Dk], fp32, value-column major).  A
+// portion that starts at position 0 reads neither; every portion leaves both at its end.
+//
+// delta_prep_kernel: a workgroup per token.  Convolution + silu of every channel into LDS (inputs from
+//   the portion's rows, then from the tail, zeros before position 0); a wave per q / k group forms both
+//   unit vectors and k . q; fp32 rows out: [q | k] per group, v, the decays, (beta | k . q).  Batches of one
+//   row per sequence advance the tail in the same launch (a thread owns its channels), other batches in
+//   delta_tail_kernel afterwards, since rows of a portion read the old tail.
+// delta_scan_kernel: workgroup = (sequence portion, head, slice of value columns).  The columns of S are
+//   independent chains: column c needs a_c = (g S_c) . k and b_c = (g S_c) . q, then u_c = beta (v_c - a_c),
+//   S_c <- g S_c + k u_c, and o_c = b_c + u_c (k . q), which is S_c . q after the write.  A column's Dk
+//   entries sit in the registers of P lanes (R each, rows interleaved over the lanes), C columns a thread;
+//   tokens are staged through LDS in chunks; a_c and b_c are reduced over the P lanes by shuffles.  A
+//   decode batch is the same launch with one-token portions.
+// delta_out_kernel: the per-head unit norm, its weight and the gate; a wave per (token, head).
+#include "common.h"
+
+namespace la {
+
+constexpr int DR_NT = 256;
+constexpr int DR_TC = 16;        // tokens staged per chunk
+constexpr int DR_MAXTAPS = 16;
+
+LA_DEV float dr_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+LA_DEV int portion_of(const int* __restrict__ cu_q, int nseq, int t) {
+  int lo = 0, hi = nseq - 1;       // cu_q[seq] <= t < cu_q[seq + 1]
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+template <typename AT>
+__global__ __launch_bounds__(DR_NT) void delta_prep_kernel(
+    const AT* __restrict__ src, long ld, const AT* __restrict__ dec, int H, int G, int Dk, int Dv, int taps,
+    const float* __restrict__ w, const float* __restrict__ dt_bias, const float* __restrict__ a_log, float unit_eps,
+    const int* __restrict__ pos, const int* __restrict__ cu_q, int nseq, const int* __restrict__ sslots,
+    AT* __restrict__ tail, int single, float* __restrict__ qk, float* __restrict__ vf, float* __restrict__ gd,
+    float* __restrict__ bq) {
+  extern __shared__ float cv[];        // [C] convolved, activated channels of this token
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int Cqk = G * Dk, Cv = H * Dv, C = 2 * Cqk + Cv;
+  const int seq = single ? t : portion_of(cu_q, nseq, t);
+  const int a = cu_q[seq], p = pos[t], p0 = pos[a];
+  const int slot = sslots[seq];
+  const AT* st = (slot >= 0 && taps > 1) ? tail + (long)slot * (taps - 1) * C : nullptr;
+  for (int c = tid; c < C; c += DR_NT) {
+    float acc = 0.f;
+    float cur[DR_MAXTAPS];             // this channel's inputs at positions p - taps + 1 .. p
+#pragma unroll
+    for (int j = 0; j < DR_MAXTAPS; ++j) {
+      if (j < taps) {
+        const int pj = p - (taps - 1) + j;
+        float v = 0.f;
+        if (pj >= p0) v = (float)src[(long)(a + pj - p0) * ld + c];
+        else if (pj >= 0 && st) v = (float)st[(long)(pj - p0 + taps - 1) * C + c];
+        cur[j] = v;
+        acc = fmaf(w[(long)c * taps + j], v, acc);
+      }
+    }
+    const float y = acc / (1.f + expf(-acc));
+    cv[c] = y;
+    if (c >= 2 * Cqk) vf[(long)t * Cv + (c - 2 * Cqk)] = y;
+    if (single && slot >= 0 && taps > 1) {      // one row per sequence: the tail moves on by one position
+      AT* sw = tail + (long)slot * (taps - 1) * C;
+#pragma unroll
+      for (int j = 1; j < DR_MAXTAPS; ++j)
+        if (j < taps) sw[(long)(j - 1) * C + c] = (AT)cur[j];
+    }
+  }
+  __syncthreads();
+  const float qscale = 1.f / sqrtf((float)Dk);
+  for (int g = wave; g < G; g += DR_NT / 64) {
+    const float* q = cv + (long)g * Dk;
+    const float* k = cv + Cqk + (long)g * Dk;
+    float sq = 0.f, sk = 0.f, dot = 0.f;
+    for (int d = lane; d < Dk; d += 64) {
+      sq = fmaf(q[d], q[d], sq);
+      sk = fmaf(k[d], k[d], sk);
+      dot = fmaf(q[d], k[d], dot);
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    dot = wave_sum(dot);
+    const float iq = qscale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
+    float* qo = qk + ((long)t * 2 * G + g) * Dk;
+    float* ko = qo + (long)G * Dk;
+    for (int d = lane; d < Dk; d += 64) {
+      qo[d] = q[d] * iq;
+      ko[d] = k[d] * ik;
+    }
+    if (lane == 0) bq[(long)t * (H + G) + H + g] = dot * iq * ik;
+  }
+  for (int h = tid; h < H; h += DR_NT) {
+    const float b = (float)src[(long)t * ld + C + h];
+    bq[(long)t * (H + G) + h] = 1.f / (1.f + expf(-b));
+  }
+  for (int e = tid; e < H * Dk; e += DR_NT) {
+    const int h = e / Dk;
+    const float dt = dr_softplus((float)dec[(long)t * H * Dk + e] + dt_bias[e]);
+    gd[(long)t * H * Dk + e] = expf(-expf(a_log[h]) * dt);
+  }
+}
+
+// tail row i of a sequence <- the input at position end - (taps - 1) + i: a row of this portion, an
+// older tail row, or zero before position 0.  A thread per (sequence, channel) reads all, then writes.
+template <typename AT>
+__global__ __launch_bounds__(DR_NT) void delta_tail_kernel(const AT* __restrict__ src, long ld, int C, int taps,
+                                                           const int* __restrict__ pos, const int* __restrict__ cu_q,
+                                                           const int* __restrict__ sslots, AT* __restrict__ tail) {
+  const int seq = blockIdx.x, c = blockIdx.y * DR_NT + threadIdx.x;
+  if (c >= C) return;
+  const int a = cu_q[seq], n = cu_q[seq + 1] - a, slot = sslots[seq];
+  if (n <= 0 || slot < 0) return;
+  const int p0 = pos[a], pend = p0 + n;
+  AT* st = tail + (long)slot * (taps - 1) * C;
+  AT nv[DR_MAXTAPS];
+#pragma unroll
+  for (int i = 0; i < DR_MAXTAPS - 1; ++i) {
+    if (i < taps - 1) {
+      const int pi = pend - (taps - 1) + i;
+      AT v = (AT)0.f;
+      if (pi >= p0) v = src[(long)(a + pi - p0) * ld + c];
+      else if (pi >= 0) v = st[(long)(pi - p0 + taps - 1) * C + c];
+      nv[i] = v;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DR_MAXTAPS - 1; ++i)
+    if (i < taps - 1) st[(long)i * C + c] = nv[i];
+}
+
+template <int R, int C>
+__global__ __launch_bounds__(DR_NT) void delta_scan_kernel(
+    const float* __restrict__ qk, const float* __restrict__ vf, const float* __restrict__ gd, const float* __restrict__ bq,
+    int H, int G, int Dk, int Dv, const int* __restrict__ pos, const int* __restrict__ cu_q,
+    const int* __restrict__ sslots, float* __restrict__ state, float* __restrict__ o, int P) {
+  extern __shared__ float lds[];
+  const int DkP = P * R;                 // padded key width (rows beyond Dk hold zeros)
+  const int cpw = DR_NT / P * C;         // value columns of this workgroup
+  float* qs = lds;                       // [TC][DkP]
+  float* ks = qs + DR_TC * DkP;          // [TC][DkP]
+  float* gs = ks + DR_TC * DkP;          // [TC][DkP]
+  float* vs = gs + DR_TC * DkP;          // [TC][cpw]
+  float* bs = vs + DR_TC * cpw;          // [TC][2]: beta, k . q
+  const int seq = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * cpw;
+  const int tid = threadIdx.x, part = tid % P, cg = tid / P, cb = c0 + cg * C;   // this thread's first column
+  const int a = cu_q[seq], b = cu_q[seq + 1];
+  if (b <= a) return;
+  const int slot = sslots[seq];
+  float* st = slot >= 0 ? state + (((long)slot * H + h) * Dv + cb) * Dk : nullptr;
+  const bool zero = pos[a] == 0;
+  const int g = h / (H / G);
+  float S[C][R];
+#pragma unroll
+  for (int ci = 0; ci < C; ++ci)
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int r = j * P + part;
+      S[ci][j] = (st && !zero && r < Dk && cb + ci < Dv) ? st[(long)ci * Dk + r] : 0.f;
+    }
+  for (int t0 = a; t0 < b; t0 += DR_TC) {
+    const int n = min(DR_TC, b - t0);
+    __syncthreads();
+    for (int e = tid; e < n * DkP; e += DR_NT) {
+      const int tt = e / DkP, d = e - tt * DkP;
+      float qv = 0.f, kv = 0.f, gv = 1.f;
+      if (d < Dk) {
+        const float* row = qk + ((long)(t0 + tt) * 2 * G + g) * Dk + d;
+        qv = row[0];
+        kv = row[(long)G * Dk];
+        gv = gd[((long)(t0 + tt) * H + h) * Dk + d];
+      }
+      qs[e] = qv;
+      ks[e] = kv;
+      gs[e] = gv;
+    }
+    for (int e = tid; e < n * cpw; e += DR_NT) {
+      const int tt = e / cpw, cc = e - tt * cpw;
+      vs[e] = (c0 + cc < Dv) ? vf[((long)(t0 + tt) * H + h) * Dv + c0 + cc] : 0.f;
+    }
+    if (tid < n) {
+      bs[2 * tid] = bq[(long)(t0 + tid) * (H + G) + h];
+      bs[2 * tid + 1] = bq[(long)(t0 + tid) * (H + G) + H + g];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < n; ++tt) {
+      const float beta = bs[2 * tt], kq = bs[2 * tt + 1];
+      float ak[C], aq[C];
+#pragma unroll
+      for (int ci = 0; ci < C; ++ci) ak[ci] = aq[ci] = 0.f;
+      const float* kr = ks + tt * DkP + part;
+      const float* qr = qs + tt * DkP + part;
+      const float* gr = gs + tt * DkP + part;
+      float kj[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        kj[j] = kr[j * P];
+        const float qj = qr[j * P], gj = gr[j * P];
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) {
+          const float s = gj * S[ci][j];
+          S[ci][j] = s;
+          ak[ci] = fmaf(s, kj[j], ak[ci]);
+          aq[ci] = fmaf(s, qj, aq[ci]);
+        }
+      }
+#pragma unroll
+      for (int ci = 0; ci < C; ++ci) {
+        float x = ak[ci], y = aq[ci];
+        for (int w = P >> 1; w > 0; w >>= 1) {
+          x += __shfl_xor(x, w, 64);
+          y += __shfl_xor(y, w, 64);
+        }
+        const float u = beta * (vs[tt * cpw + cg * C + ci] - x);
+#pragma unroll
+        for (int j = 0; j < R; ++j) S[ci][j] = fmaf(kj[j], u, S[ci][j]);
+        if (part == 0 && cb + ci < Dv) o[((long)(t0 + tt) * H + h) * Dv + cb + ci] = fmaf(u, kq, y);
+      }
+    }
+  }
+  if (st) {
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci)
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const int r = j * P + part;
+        if (r < Dk && cb + ci < Dv) st[(long)ci * Dk + r] = S[ci][j];
+      }
+  }
+}
+
+// out[t][h][d] = o / sqrt(mean(o^2) + eps) * w[d] * sigmoid(gate): a wave per (token, head)
+template <typename AT>
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o, const AT* __restrict__ gate, int Dv,
+                                                        long rows, int H, const float* __restrict__ w, float eps,
+                                                        AT* __restrict__ out) {
+  const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const float* orow = o + r * Dv;
+  float ss = 0.f;
+  for (int d = lane; d < Dv; d += 64) ss = fmaf(orow[d], orow[d], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)Dv + eps);
+  for (int d = lane; d < Dv; d += 64) {
+    const float gv = (float)gate[r * Dv + d];
+    out[r * Dv + d] = (AT)(orow[d] * inv * w[d] / (1.f + expf(-gv)));
+  }
+}
+
+template <typename AT>
+static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, int T, int nseq, int H, int G, int Dk, int Dv,
+                        int taps, const float* w, const float* dt_bias, const float* a_log, const float* nw, float eps,
+                        float unit_eps, const int* pos, const int* cu_q, const int* sslots, AT* tail, float* state,
+                        int single, float* qk, float* vf, float* gd, float* bq, float* o, AT* out, hipStream_t st) {
+  const int C = 2 * G * Dk + H * Dv;
+  const size_t shm0 = (size_t)C * sizeof(float);
+  if (shm0 > 150 * 1024) return -6;
+  if (shm0 > 48 * 1024)
+    (void)hipFuncSetAttribute((const void*)delta_prep_kernel<AT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm0);
+  hipLaunchKernelGGL(delta_prep_kernel<AT>, dim3(T), dim3(DR_NT), shm0, st, src, ld, dec, H, G, Dk, Dv, taps, w, dt_bias,
+                     a_log, unit_eps, pos, cu_q, nseq, sslots, tail, single, qk, vf, gd, bq);
+  if (!single && taps > 1)
+    hipLaunchKernelGGL(delta_tail_kernel<AT>, dim3(nseq, (C + DR_NT - 1) / DR_NT), dim3(DR_NT), 0, st, src, ld, C, taps, pos,
+                       cu_q, sslots, tail);
+  // P lanes per group of Cc value columns (power of two), R rows per lane: P * R >= Dk; a thread keeps
+  // Cc x R state entries.  More lanes per group while the launch has fewer than about four workgroups
+  // per compute unit: a scan is a chain of dependent steps, so resident waves hide its latencies.
+  const int Cc = Dv >= 64 ? 4 : 1;
+  int P = 8;
+  while (P < 64 && (Dk + P - 1) / P > (Cc == 4 ? 8 : 16)) P <<= 1;
+  if ((Dk + P - 1) / P > 16) return -5;
+  while (P < 64 && (Dk + P - 1) / P > 2 && (long)nseq * H * ((Dv + DR_NT / P * Cc - 1) / (DR_NT / P * Cc)) < 1024) P <<= 1;
+  const int need = (Dk + P - 1) / P;
+  const int cpw = DR_NT / P * Cc;
+  const int nz = (Dv + cpw - 1) / cpw;
+#define LA_DR_LAUNCH(RR, CC)                                                                                         \
+  {                                                                                                                  \
+    const size_t shm = (size_t)(3 * DR_TC * P * RR + DR_TC * cpw + 2 * DR_TC) * sizeof(float);                       \
+    if (shm > 150 * 1024) return -6;                                                                                 \
+    if (shm > 48 * 1024)                                                                                             \
+      (void)hipFuncSetAttribute((const void*)delta_scan_kernel<RR, CC>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                (int)shm);                                                                           \
+    hipLaunchKernelGGL((delta_scan_kernel<RR, CC>), dim3(nseq, H, nz), dim3(DR_NT), shm, st, (const float*)qk,       \
+                       (const float*)vf, (const float*)gd, (const float*)bq, H, G, Dk, Dv, pos, cu_q, sslots, state, \
+                       o, P);                                                                                        \
+  }
+#define LA_DR_R(CC)                                                                                                  \
+  {                                                                                                                  \
+    if (need <= 1) LA_DR_LAUNCH(1, CC)                                                                               \
+    else if (need <= 2) LA_DR_LAUNCH(2, CC)                                                                          \
+    else if (need <= 4) LA_DR_LAUNCH(4, CC)                                                                          \
+    else if (need <= 8) LA_DR_LAUNCH(8, CC)                                                                          \
+    else LA_DR_LAUNCH(16, CC)                                                                                        \
+  }
+  if (Cc == 4) LA_DR_R(4)
+  else LA_DR_R(1)
+#undef LA_DR_R
+#undef LA_DR_LAUNCH
+  const long rows = (long)T * H;
+  hipLaunchKernelGGL(delta_out_kernel<AT>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const float*)o, gate, Dv,
+                     rows, H, nw, eps, out);
+  return (int)hipGetLastError();
+}
+
+}  // namespace la
+
+extern "C" int la_delta_rule(int f32, const void* src, long ld, const void* dec, const void* gate, int T, int nseq, int H,
+                             int G, int Dk, int Dv, int taps, int nslots, const void* conv_w, const void* dt_bias,
+                             const void* a_log, const void* norm_w, float eps, float unit_eps, const void* pos,
+                             const void* cu_q, const void* sslots, void* tail, void* state, int single, void* qk, void* vf,
+                             void* gd, void* bq, void* o, void* out, void* stream) {
+  using namespace la;
+  if (T <= 0 || nseq <= 0 || H <= 0 || G <= 0 || H % G || Dk <= 0 || Dv <= 0 || taps < 1 || taps > DR_MAXTAPS ||
+      nslots <= 0 || ld < 2L * G * Dk + (long)H * Dv + H)
+    return -1;
+  if (!src || !dec || !gate || !conv_w || !dt_bias || !a_log || !norm_w || !pos || !cu_q || !sslots || !state || !qk ||
+      !vf || !gd || !bq || !o || !out || (taps > 1 && !tail))
+    return -2;
+  if (single && T != nseq) return -3;
+  hipStream_t st = (hipStream_t)stream;
+  if (f32)
+    return delta_launch<float>((const float*)src, ld, (const float*)dec, (const float*)gate, T, nseq, H, G, Dk, Dv, taps,
+                               (const float*)conv_w, (const float*)dt_bias, (const float*)a_log, (const float*)norm_w, eps,
+                               unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (float*)tail,
+                               (float*)state, single, (float*)qk, (float*)vf, (float*)gd, (float*)bq, (float*)o,
+                               (float*)out, st);
+  return delta_launch<bf16>((const bf16*)src, ld, (const bf16*)dec, (const bf16*)gate, T, nseq, H, G, Dk, Dv, taps,
+                            (const float*)conv_w, (const float*)dt_bias, (const float*)a_log, (const float*)norm_w, eps,
+                            unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (bf16*)tail, (float*)state,
+                            single, (float*)qk, (float*)vf, (float*)gd, (float*)bq, (float*)o, (bf16*)out, st);
+}

@@ -230,7 +230,127 @@ __global__ __launch_bounds__(256) void side_gate_kernel(RowSrc src, int n, long 
   put(out, out_f32, e, gelu_tanh_f(src_at(src, e)) * emb);
 }
 
+// Pre-normed streams whose norm works on groups:  res += branch;  out = res, each of `groups` equal
+// consecutive parts divided by its own sqrt(mean(part^2) + eps), times w.  A workgroup per row; after
+// the add every wave takes whole groups (group g -> wave g mod 4), so a group's statistics need no
+// workgroup-wide reduction; the row is re-read from cache.
+__global__ __launch_bounds__(NC_NT) void add_group_norm_kernel(float* __restrict__ res, int D, RowSrc src, int has_src,
+                                                               const float* __restrict__ w, float eps, int groups,
+                                                               void* __restrict__ out, int out_f32) {
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const long base = (long)t * D;
+  if (has_src) {
+    for (int c = tid; c < D; c += NC_NT) res[base + c] += src_at(src, base + c);
+    __syncthreads();
+  }
+  const int gs = D / groups, wave = tid >> 6, lane = tid & 63;
+  for (int g = wave; g < groups; g += NC_NT / 64) {
+    const float* row = res + base + (long)g * gs;
+    float ss = 0.f;
+    for (int c = lane; c < gs; c += 64) ss = fmaf(row[c], row[c], ss);
+    const float inv = 1.f / sqrtf(wave_sum(ss) / (float)gs + eps);
+    for (int c = lane; c < gs; c += 64) put(out, out_f32, base + (long)g * gs + c, row[c] * inv * w[g * gs + c]);
+  }
+}
+
+// one group and few groups of wide rows: the whole workgroup per group (block reductions)
+__global__ __launch_bounds__(NC_NT) void add_group_norm_wide_kernel(float* __restrict__ res, int D, RowSrc src, int has_src,
+                                                                    const float* __restrict__ w, float eps, int groups,
+                                                                    void* __restrict__ out, int out_f32) {
+  __shared__ float red[NC_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const long base = (long)t * D;
+  const int gs = D / groups;
+  for (int g = 0; g < groups; ++g) {
+    float ss = 0.f;
+    for (int c = g * gs + tid; c < (g + 1) * gs; c += NC_NT) {
+      float x = res[base + c];
+      if (has_src) {
+        x += src_at(src, base + c);
+        res[base + c] = x;
+      }
+      ss = fmaf(x, x, ss);
+    }
+    const float inv = 1.f / sqrtf(block_sum<NC_NT>(ss, red) / (float)gs + eps);
+    for (int c = g * gs + tid; c < (g + 1) * gs; c += NC_NT) put(out, out_f32, base + c, res[base + c] * inv * w[c]);
+  }
+}
+
+// y = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e over a row of F values (rms with eps inside
+// the root): a workgroup per row, one pass for the three sums of even powers, one for the outputs
+__global__ __launch_bounds__(NC_NT) void poly_norm_act_kernel(RowSrc src, int F, const float* __restrict__ coef, float eps,
+                                                              void* __restrict__ out, int out_f32) {
+  __shared__ float red[NC_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const long base = (long)t * F;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int c = tid; c < F; c += NC_NT) {
+    const float z = src_at(src, base + c), z2 = z * z;
+    s2 += z2;
+    s4 = fmaf(z2, z2, s4);
+    s6 = fmaf(z2 * z2, z2, s6);
+  }
+  s2 = block_sum<NC_NT>(s2, red);
+  s4 = block_sum<NC_NT>(s4, red);
+  s6 = block_sum<NC_NT>(s6, red);
+  const float i1 = coef[0] / sqrtf(s2 / (float)F + eps), i2 = coef[1] / sqrtf(s4 / (float)F + eps),
+              i3 = coef[2] / sqrtf(s6 / (float)F + eps), e = coef[3];
+  for (int c = tid; c < F; c += NC_NT) {
+    const float z = src_at(src, base + c);
+    put(out, out_f32, base + c, fmaf(z, i1, fmaf(z * z, i2, fmaf(z * z * z, i3, e))));
+  }
+}
+
+// out = x * sigmoid(gate), gate rows with their own stride (columns of a wider projection)
+__global__ __launch_bounds__(256) void sigmoid_mul_kernel(const void* __restrict__ x, int x_f32, const void* __restrict__ g,
+                                                          int g_f32, long ldg, int N, long total, void* __restrict__ out,
+                                                          int out_f32) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long t = e / N;
+  const int c = (int)(e - t * N);
+  const float xv = x_f32 ? ((const float*)x)[e] : (float)((const bf16*)x)[e];
+  const float gv = g_f32 ? ((const float*)g)[t * ldg + c] : (float)((const bf16*)g)[t * ldg + c];
+  put(out, out_f32, e, xv / (1.f + expf(-gv)));
+}
+
 }  // namespace la
+
+extern "C" int la_add_group_norm(void* res, int T, int D, const void* sp, int src_f32, long slab, int S, const void* w,
+                                 float eps, int groups, void* out, int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || D <= 0 || groups < 1 || D % groups || !res || !w || !out) return -1;
+  const int has = sp != nullptr;
+  if (has && src_f32 && S < 1) return -4;
+  RowSrc s{sp, src_f32, slab, S};
+  if (groups >= 4 && D / groups <= 1024)
+    hipLaunchKernelGGL(add_group_norm_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, (float*)res, D, s, has,
+                       (const float*)w, eps, groups, out, out_f32);
+  else
+    hipLaunchKernelGGL(add_group_norm_wide_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, (float*)res, D, s, has,
+                       (const float*)w, eps, groups, out, out_f32);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_poly_norm_act(const void* sp, int src_f32, long slab, int S, int T, int F, const void* coef, float eps,
+                                void* out, int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || F <= 0 || !sp || !coef || !out) return -1;
+  RowSrc s{sp, src_f32, slab, S};
+  hipLaunchKernelGGL(poly_norm_act_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, s, F, (const float*)coef, eps, out,
+                     out_f32);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_sigmoid_mul(const void* x, int x_f32, const void* g, int g_f32, long ldg, int T, int N, void* out,
+                              int out_f32, void* stream) {
+  using namespace la;
+  if (T <= 0 || N <= 0 || !x || !g || !out || ldg < N) return -1;
+  const long total = (long)T * N;
+  hipLaunchKernelGGL(sigmoid_mul_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, x_f32,
+                     g, g_f32, ldg, N, total, out, out_f32);
+  return (int)hipGetLastError();
+}
 
 extern "C" int la_norm_chain(void* res, int T, int D, const void* sp, int src_f32, long slab, int S, int post, float pa,
                              const void* pw, const void* pb, float eps, const void* addv, int replace, int pre, float qa,

@@ -161,7 +161,124 @@ __global__ __launch_bounds__(256) void sinusoid_add_kernel(float* __restrict__ r
   }
 }
 
+// A workgroup per token: per-head RMS norm with a weight on q and k (a wave per head), rotation of their
+// first `rot` dims in the (i, i + rot / 2) layout, values rotated over their whole width with their own
+// frequency table (vfreqs null: values pass), q -> q_out, K / V -> pages.
+template <typename AT>
+__global__ __launch_bounds__(RP_NT) void qk_norm_rope_pages_kernel(
+    const AT* __restrict__ src, long ld, int H, int D, int G, int Dv, const int* __restrict__ pos,
+    const int* __restrict__ slots, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const float* __restrict__ freqs, float mag, int rot, const float* __restrict__ vfreqs, AT* __restrict__ q_out,
+    AT* __restrict__ kc, AT* __restrict__ vc, int BS) {
+  extern __shared__ float cs[];          // [rot / 2][2] for q / k, then [Dv / 2][2] for v
+  float* vcs = cs + rot;
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int Cq = H * D, Ck = G * D, Cv = G * Dv, half = rot >> 1, vhalf = Dv >> 1;
+  const AT* row = src + (long)t * ld;
+  const int p = pos[t];
+  fill_cos_sin(cs, rot, p, freqs, mag);
+  if (vfreqs) fill_cos_sin(vcs, Dv, p, vfreqs, 1.f);
+  __syncthreads();
+  const int slot = slots[t];
+  const int blk = slot >= 0 ? slot / BS : 0, off = slot >= 0 ? slot - blk * BS : 0;
+  for (int u = wave; u < H + G; u += RP_NT / 64) {
+    const bool isq = u < H;
+    if (!isq && slot < 0) continue;
+    const AT* x = isq ? row + (long)u * D : row + Cq + (long)(u - H) * D;
+    const float* w = isq ? qw : kw;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const float v = (float)x[d];
+      ss = fmaf(v, v, ss);
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+    AT* dst = isq ? q_out + (long)t * Cq + (long)u * D : kc + (((long)blk * G + (u - H)) * BS + off) * D;
+    for (int d = lane; d < D; d += 64) {
+      float y;
+      if (d < rot) {
+        const bool first = d < half;
+        const int i = first ? d : d - half;
+        const float a = (float)x[i] * inv * w[i], b = (float)x[i + half] * inv * w[i + half];
+        const float c = cs[2 * i], sn = cs[2 * i + 1];
+        y = first ? a * c - b * sn : b * c + a * sn;
+      } else {
+        y = (float)x[d] * inv * w[d];
+      }
+      dst[d] = (AT)y;
+    }
+  }
+  if (slot < 0) return;
+  for (int e = tid; e < Cv; e += RP_NT) {
+    const int g = e / Dv, d = e - g * Dv;
+    const AT* x = row + Cq + Ck + (long)g * Dv;
+    AT y = x[d];
+    if (vfreqs) {
+      const bool first = d < vhalf;
+      const int i = first ? d : d - vhalf;
+      const float a = (float)x[i], b = (float)x[i + vhalf], c = vcs[2 * i], sn = vcs[2 * i + 1];
+      y = (AT)(first ? a * c - b * sn : b * c + a * sn);
+    }
+    vc[((((long)blk * G + g) * (BS >> 3) + (off >> 3)) * Dv + d) * 8 + (off & 7)] = y;
+  }
+}
+
+// every head of a row turned over its whole width, dims m and m + Dv / 2 by sign * pos * freqs[m], times scale
+template <typename AT>
+__global__ __launch_bounds__(RP_NT) void rotate_heads_kernel(const AT* __restrict__ x, int H, int Dv,
+                                                             const int* __restrict__ pos, const float* __restrict__ freqs,
+                                                             float sign, float scale, AT* __restrict__ out, long ldo) {
+  extern __shared__ float cs[];          // [Dv / 2][2]
+  const int t = blockIdx.x, vhalf = Dv >> 1;
+  for (int i = threadIdx.x; i < vhalf; i += RP_NT) {
+    const float a = sign * ((float)pos[t] * freqs[i]);
+    cs[2 * i] = cosf(a) * scale;
+    cs[2 * i + 1] = sinf(a) * scale;
+  }
+  __syncthreads();
+  const AT* row = x + (long)t * H * Dv;
+  for (int e = threadIdx.x; e < H * vhalf; e += RP_NT) {
+    const int h = e / vhalf, i = e - h * vhalf;
+    const float a = (float)row[h * Dv + i], b = (float)row[h * Dv + i + vhalf], c = cs[2 * i], sn = cs[2 * i + 1];
+    out[(long)t * ldo + h * Dv + i] = (AT)(a * c - b * sn);
+    out[(long)t * ldo + h * Dv + i + vhalf] = (AT)(b * c + a * sn);
+  }
+}
+
 }  // namespace la
+
+extern "C" int la_qk_norm_rope_pages(int f32, const void* src, long ld, int T, int H, int D, int G, int Dv, const void* pos,
+                                     const void* slots, const void* qw, const void* kw, float eps, const void* freqs,
+                                     float mag, int rot, const void* vfreqs, void* q_out, void* kc, void* vc, int BS,
+                                     void* stream) {
+  using namespace la;
+  if (T <= 0 || H <= 0 || D <= 0 || G <= 0 || Dv <= 0 || (rot & 1) || rot < 0 || rot > D || (vfreqs && (Dv & 1))) return -1;
+  if (ld < (long)(H + G) * D + (long)G * Dv || BS <= 0 || (BS & 7)) return -2;
+  if (!src || !pos || !slots || !qw || !kw || !freqs || !q_out || !kc || !vc) return -3;
+  const size_t shm = (size_t)(rot + Dv + 2) * sizeof(float);
+  if (f32)
+    hipLaunchKernelGGL(qk_norm_rope_pages_kernel<float>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const float*)src,
+                       ld, H, D, G, Dv, (const int*)pos, (const int*)slots, (const float*)qw, (const float*)kw, eps,
+                       (const float*)freqs, mag, rot, (const float*)vfreqs, (float*)q_out, (float*)kc, (float*)vc, BS);
+  else
+    hipLaunchKernelGGL(qk_norm_rope_pages_kernel<bf16>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const bf16*)src, ld,
+                       H, D, G, Dv, (const int*)pos, (const int*)slots, (const float*)qw, (const float*)kw, eps,
+                       (const float*)freqs, mag, rot, (const float*)vfreqs, (bf16*)q_out, (bf16*)kc, (bf16*)vc, BS);
+  return (int)hipGetLastError();
+}
+
+extern "C" int la_rotate_heads(int f32, const void* x, int T, int H, int Dv, const void* pos, const void* freqs, float sign,
+                               float scale, void* out, long ldo, void* stream) {
+  using namespace la;
+  if (T <= 0 || H <= 0 || Dv <= 0 || (Dv & 1) || ldo < (long)H * Dv || !x || !pos || !freqs || !out) return -1;
+  const size_t shm = (size_t)(Dv + 2) * sizeof(float);
+  if (f32)
+    hipLaunchKernelGGL(rotate_heads_kernel<float>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const float*)x, H, Dv,
+                       (const int*)pos, (const float*)freqs, sign, scale, (float*)out, ldo);
+  else
+    hipLaunchKernelGGL(rotate_heads_kernel<bf16>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const bf16*)x, H, Dv,
+                       (const int*)pos, (const float*)freqs, sign, scale, (bf16*)out, ldo);
+  return (int)hipGetLastError();
+}
 
 extern "C" int la_qk_norm_pages(int f32, const void* src, int ld, int T, int H, int Dq, int G, int Dk, int Dv,
                                 const void* pos, const void* slots, float eps, float coef, int every, void* q_out,
