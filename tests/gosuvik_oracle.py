@@ -216,17 +216,26 @@ def poly_ff(W, p, h, eps):
 
 
 def router(W, p, f, h):
-    """(chosen experts [T, top], their weights [T, top], margin between the last chosen and the first left out)."""
-    s = torch.softmax(h @ W[p + "router"].T, -1)
+    """(chosen experts [T, top], their weights [T, top], margin [T]: the last chosen logit minus the first one
+    left out, in units of the logits' spread; infinite when every expert is chosen)."""
+    z = h @ W[p + "router"].T
+    s = torch.softmax(z, -1)
     top = f["router"]["top"]
     val, idx = torch.sort(s, dim=-1, descending=True, stable=True)
     w = val[:, :top] / (val[:, :top].sum(-1, keepdim=True) + 1e-20)
-    margin = val[:, top - 1] - val[:, top] if top < s.shape[1] else torch.full((h.shape[0],), 1.0, dtype=F64)
+    if top < s.shape[1]:
+        zs = torch.sort(z, dim=-1, descending=True).values
+        margin = (zs[:, top - 1] - zs[:, top]) / z.std(-1).clamp_min(1e-9)
+    else:
+        margin = torch.full((h.shape[0],), float("inf"), dtype=F64)
     return idx[:, :top], w, margin
 
 
-def expert_ff(W, p, f, h):
-    ids, w, _ = router(W, p, f, h)
+def expert_ff(W, p, f, h, margins=None):
+    ids, w, margin = router(W, p, f, h)
+    if margins is not None:
+        for t in range(h.shape[0]):
+            margins[t] = min(margins[t], float(margin[t]))
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F64)
     for t in range(h.shape[0]):
         for e, we in zip(ids[t].tolist(), w[t]):
@@ -245,8 +254,9 @@ def runs(cfg):
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def forward(cfg, W, tokens, streams=None):
-    """float64 logits [T, vocab] of one sequence; streams (a list) receives x after every layer run."""
+def forward(cfg, W, tokens, streams=None, margins=None):
+    """float64 logits [T, vocab] of one sequence; streams (a list) receives x after every layer run;
+    margins (a list of T floats) is lowered to every position's smallest router margin."""
     W = {k: v.to(F64) for k, v in W.items()}
     eps, groups = cfg["norm"]["eps"], cfg["norm"].get("groups", 1)
     x = W["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -257,7 +267,7 @@ def forward(cfg, W, tokens, streams=None):
         f = L.get("mlp")
         if f:
             hn = group_norm(x, W[p + "norm2"], eps, groups)
-            x = x + (poly_ff(W, p + "mlp.", hn, eps) if f["kind"] == "dense" else expert_ff(W, p + "mlp.", f, hn))
+            x = x + (poly_ff(W, p + "mlp.", hn, eps) if f["kind"] == "dense" else expert_ff(W, p + "mlp.", f, hn, margins))
         if streams is not None:
             streams.append(x.clone())
     return group_norm(x, W["final.norm"], eps, groups) @ W["head"].T

@@ -1,0 +1,531 @@
+"""Gosuvik through the framework (reader, model class, K/V pools per layer run, convolution and
+recurrent state slots, native scheduler, schedule replay, generation) against the plain oracle of
+tests/gosuvik_oracle.py.
+
+Every test builds its own small random checkpoint.  The CPU runs use the operator layer's PyTorch
+paths; the `gpu` runs put the same engine on the HIP kernels, in bf16 and in fp32.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import gosuvik_oracle as oracle
+from localai_amd.engine.llm_engine import EngineConfig, LLMEngine
+from localai_amd.engine.sampling_params import SamplingParams
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+MODES = [("cpu", "float32"), ("cpu", "bfloat16"),
+         pytest.param("cuda:0", "float32", marks=pytest.mark.gpu), pytest.param("cuda:0", "bfloat16", marks=pytest.mark.gpu)]
+
+# a router margin (last chosen logit minus the first one left out, in units of the logits' spread) below
+# which 16-bit rounding upstream may decide the choice
+MARGIN = 0.1
+YARN = {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.0}
+
+
+def delta(heads=4, kv=2, dim=8, vdim=6, conv=3, ra=5, rg=7):
+    return {"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "conv": conv},
+            "ranks": (ra, rg)}
+
+
+def latent(heads=3, dim=8, rot_dim=4, vdim=6, rank=10, window=12, base=100.0, scaling=YARN, scale=0.3):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": rank, "scale": scale,
+         "rot": {"dims": rot_dim, "base": base}}
+    if scaling:
+        m["rot"]["scaling"] = scaling
+    if window:
+        m["mask"] = {"size": window}
+    return {"type": "latent_attention", "mixer": m}
+
+
+def parallel(heads=4, kv=2, dim=12, vdim=8, rot=8, window=9, factor=4.0, base=50.0, scale=0.3, r_heads=2, r_dim=6, r_vdim=10,
+             cap=8.0, ls=0.7, rs=0.4):
+    left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale, "rot": {"dims": rot, "base": base}}
+    if factor:
+        left["rot"]["scaling"] = {"factor": factor}
+    if window:
+        left["mask"] = {"size": window}
+    right = {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "gate_cap": cap}
+    return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": ls, "right_scale": rs}}
+
+
+def dense(layer, n=40):
+    return dict(layer, mlp={"kind": "dense", "ff": n} if n else None)
+
+
+def moe(layer, experts=5, top=2, n=24):
+    return dict(layer, mlp={"kind": "moe", "expert": {"ff": n}, "router": {"experts": experts, "top": top}})
+
+
+# layer orders and sizes unlike one another: norm groups 1 / several, a loop over the middle / the
+# whole model / none, q / k heads of the delta rule fewer than / equal to its heads, 1 to 5 taps, key
+# width = / != value width everywhere, windows shorter than a page / longer than the prompts / none,
+# rotation over a part / the whole of a head, with linear scaling / YaRN / none, kv heads 1 / several /
+# = heads, top 1 / some / all experts, layers without a feed-forward, branch scales 1 and others
+CONFIGS = {
+    "small": {"vocab": 61, "width": 48, "norm": {"eps": 1e-5, "groups": 4}, "loop": {"start": 1, "stop": 3, "times": 2},
+              "layers": [dense(delta()), moe(latent()), moe(parallel(), top=1), dense(delta(heads=2, kv=2, dim=6, vdim=10, conv=2), 0)]},
+    "varied": {"vocab": 83, "width": 40, "norm": {"eps": 1e-6, "groups": 1},
+               "layers": [moe(parallel(heads=6, kv=1, dim=8, vdim=12, rot=8, window=40, factor=0, r_heads=3, r_dim=10, r_vdim=4,
+                                       cap=15.0, ls=1.0, rs=1.0), experts=3, top=3, n=10),
+                          dense(latent(heads=2, dim=6, rot_dim=8, vdim=10, rank=7, window=0, scaling=None), 0),
+                          dense(delta(heads=3, kv=3, dim=10, vdim=4, conv=1, ra=3, rg=2), 24),
+                          moe(latent(heads=4, dim=4, rot_dim=2, vdim=4, rank=12, window=200, base=10000.0,
+                                     scaling={"factor": 2.0, "original": 16, "fast": 4.0, "slow": 2.0}), experts=7, top=4, n=12),
+                          dense(parallel(heads=3, kv=3, dim=6, vdim=6, rot=6, window=5, factor=8.0, r_heads=1, r_dim=12, r_vdim=12,
+                                         cap=5.0, ls=0.3, rs=1.5), 32)]},
+    "tail": {"vocab": 50, "width": 32, "norm": {"eps": 1e-5, "groups": 2}, "loop": {"start": 0, "stop": 3, "times": 3},
+             "layers": [dense(delta(heads=2, kv=1, dim=12, vdim=4, conv=5), 36),
+                        dense(parallel(heads=2, kv=1, dim=8, vdim=4, rot=4, window=17, r_heads=2, r_dim=4, r_vdim=8), 0),
+                        moe(latent(heads=2, dim=10, rot_dim=6, vdim=8, rank=6, window=16), experts=4, top=2, n=16)]},
+    # sizes no vector load likes (width % 8 != 0, odd head widths and ranks, three heads)
+    "odd": {"vocab": 51, "width": 36, "norm": {"eps": 1e-6, "groups": 3}, "loop": {"start": 2, "stop": 3, "times": 2},
+            "layers": [moe(delta(heads=3, kv=1, dim=5, vdim=7, conv=4, ra=3, rg=5), experts=3, top=2, n=13),
+                       dense(latent(heads=3, dim=5, rot_dim=6, vdim=7, rank=9, window=7), 30),
+                       moe(parallel(heads=3, kv=1, dim=10, vdim=14, rot=2, window=33, factor=3.0, r_heads=3, r_dim=7, r_vdim=9),
+                           experts=6, top=2, n=18)]},
+    # widths the GPU's specialised paths take: attention key width % 32 and value width % 16 (matrix-core
+    # tiles), equal key and value widths (the split-KV decode and prefill kernels), a latent row of 128
+    # with a latent of 96 (the latent matrix-core kernel), GEMM depths % 256 (skinny GEMMs, grouped expert
+    # GEMMs), recurrences whose state rows span several registers a lane and whose columns go four a thread
+    "wide": {"vocab": 97, "width": 256, "norm": {"eps": 1e-6, "groups": 8}, "loop": {"start": 1, "stop": 4, "times": 2},
+             "layers": [dense(delta(heads=4, kv=2, dim=64, vdim=64, conv=4, ra=16, rg=24), 512),
+                        moe(latent(heads=4, dim=32, rot_dim=32, vdim=48, rank=96, window=40, base=10000.0, scale=0.12), experts=4,
+                            top=2, n=256),
+                        moe(parallel(heads=4, kv=2, dim=64, vdim=32, rot=32, window=24, scale=0.125, r_heads=2, r_dim=64,
+                                     r_vdim=64), experts=6, top=2, n=64),
+                        dense(parallel(heads=8, kv=2, dim=64, vdim=64, rot=64, window=50, factor=2.0, scale=0.125, r_heads=4,
+                                       r_dim=32, r_vdim=96, cap=10.0), 256),
+                        dense(delta(heads=2, kv=2, dim=128, vdim=32, conv=2, ra=8, rg=8), 0)]},
+}
+
+
+def clean(cfg):
+    """The config as a checkpoint stores it (the tests' low-rank widths become shapes of tensors)."""
+    return dict(cfg, layers=[{k: v for k, v in L.items() if k != "ranks"} for L in cfg["layers"]])
+
+
+def make_weights(cfg, seed):
+    g = torch.Generator().manual_seed(seed)
+    D = cfg["width"]
+
+    def rnd(*shape, s=1.0):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    def lin(n, k, s=1.0):
+        return rnd(n, k, s=s * k ** -0.5)
+
+    def norm(n):
+        return (1.0 + 0.2 * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    W = {"embed": rnd(cfg["vocab"], D, s=0.5), "final.norm": norm(D), "head": lin(cfg["vocab"], D)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.mix.", L["mixer"]
+        W[f"l{i}.norm1"] = norm(D)
+        if L["type"] == "channel_delta":
+            H, G, dk, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+            ra, rg = L["ranks"]
+            W[p + "q"], W[p + "k"], W[p + "v"] = lin(G * dk, D, 1.5), lin(G * dk, D, 1.5), lin(H * dv, D, 1.5)
+            for n, c in (("q", G * dk), ("k", G * dk), ("v", H * dv)):
+                W[p + n + ".conv"] = rnd(c, taps, s=0.6)
+            W[p + "b"] = lin(H, D, 2.0)
+            W[p + "a1"], W[p + "a2"] = lin(ra, D), lin(H * dk, ra, 2.0)
+            W[p + "g1"], W[p + "g2"] = lin(rg, D), lin(H * dv, rg, 2.0)
+            W[p + "dt_bias"], W[p + "A_log"] = rnd(H * dk, s=1.0), (rnd(H, s=0.7).float() - 1.0).to(torch.bfloat16)
+            W[p + "norm"], W[p + "o"] = norm(dv), lin(D, H * dv)
+        elif L["type"] == "latent_attention":
+            H, dn, dr, dv, r = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            W[p + "q"], W[p + "dkv"], W[p + "dkv.norm"] = lin(H * (dn + dr), D, 1.5), lin(r + dr, D, 1.5), norm(r)
+            W[p + "uk"], W[p + "uv"] = lin(H * dn, r, 1.5), lin(H * dv, r)
+            W[p + "g"], W[p + "o"] = lin(H * dv, D, 2.0), lin(D, H * dv)
+        else:
+            l, r = m["left"], m["right"]
+            H, G, dk, dv = l["heads"], l["kv_heads"], l["dim"], l["vdim"]
+            q = p + "left."
+            W[q + "q"], W[q + "k"], W[q + "v"] = lin(H * dk, D), lin(G * dk, D), lin(G * dv, D)
+            W[q + "q.norm"], W[q + "k.norm"] = norm(dk) * 1.5, norm(dk) * 1.5
+            W[q + "sink"], W[q + "o"] = rnd(H, s=1.0), lin(D, H * dv)
+            H, dk, dv = r["heads"], r["dim"], r["vdim"]
+            q = p + "right."
+            W[q + "q"], W[q + "k"], W[q + "v"], W[q + "g"] = lin(H * dk, D), lin(H * dk, D), lin(H * dv, D), lin(H * dv, D, 2.0)
+            W[q + "i"], W[q + "f"] = lin(H, D, 2.0), lin(H, D, 2.0)
+            W[q + "i.b"], W[q + "f.b"] = rnd(H, s=1.0), (rnd(H, s=1.0).float() + 2.0).to(torch.bfloat16)
+            W[q + "norm"], W[q + "o"] = norm(H * dv), lin(D, H * dv)
+        f = L["mlp"]
+        if f:
+            p = f"l{i}.mlp."
+            W[f"l{i}.norm2"] = norm(D)
+            if f["kind"] == "dense":
+                W[p + "up"], W[p + "down"] = lin(f["ff"], D), lin(D, f["ff"])
+                W[p + "act"] = rnd(4, s=0.7)
+            else:
+                for e in range(f["router"]["experts"]):
+                    n = f["expert"]["ff"]
+                    W[p + f"e{e}.gate"], W[p + f"e{e}.up"], W[p + f"e{e}.down"] = lin(n, D), lin(n, D), lin(D, n)
+                W[p + "router"] = lin(f["router"]["experts"], D, 3.0)
+    return W
+
+
+def write_checkpoint(path, cfg, W):
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(dict(clean(cfg), architecture="Gosuvik"), f)
+    save_file({k: v.contiguous() for k, v in W.items()}, os.path.join(path, "model.safetensors"))
+
+
+_CKPT = {}
+
+
+@pytest.fixture(scope="module")
+def ckpt(tmp_path_factory):
+    def get(name, seed=0):
+        key = (name, seed)
+        if key not in _CKPT:
+            cfg = CONFIGS[name]
+            W = make_weights(cfg, seed)
+            path = str(tmp_path_factory.mktemp(f"gosuvik_{name}_{seed}"))
+            write_checkpoint(path, cfg, W)
+            _CKPT[key] = (path, clean(cfg), {k: v.float() for k, v in W.items()})
+        return _CKPT[key]
+    return get
+
+
+def engine(path, device, dtype="float32", tokens=256, slots=4, bs=16, graphs=False):
+    return LLMEngine(EngineConfig(model_path=path, device=device, context_size=tokens, max_num_seqs=slots,
+                                  max_batched_tokens=tokens, block_size=bs, max_kv_tokens=tokens, kv_pool_exact=True,
+                                  use_graphs=graphs, dtype=dtype, state_slots=slots, record_tokens=True))
+
+
+class Want:
+    """The oracle's logits of a sequence and, per position, its smallest router margin."""
+
+    def __init__(self, logits, margins):
+        self.logits, self.margins = logits, torch.tensor(margins)
+
+    def __getitem__(self, idx):
+        return Want(self.logits[idx], self.margins[idx].reshape(-1).tolist())
+
+
+def close(got, want, dtype):
+    """fp32: every position to rounding.  bf16: a position whose router margin is a close call may
+    choose other experts than the oracle (16-bit rounding of the router's input decides it), so
+    such positions count in the median only; of the others one in twenty may stand out."""
+    margins = want.margins if isinstance(want, Want) else None
+    if margins is not None:       # a choice that differs at one position changes the state every later position reads
+        margins = torch.cummin(margins, 0).values
+    want = want.logits if isinstance(want, Want) else want
+    got, want = got.detach().float().cpu(), want.float()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    err = d.pow(2).mean(-1).sqrt() / want.std(-1).clamp_min(1e-6)
+    if dtype == "float32":
+        assert float(err.max()) < 2e-4, float(err.max())
+    else:
+        sure = err if margins is None else err[margins > MARGIN]
+        worst = float(sure.max()) if sure.numel() else 0.0
+        over = int((sure > 0.12).sum())       # 16-bit rounding ahead of a sharp gate or softmax: a few positions stand out
+        assert worst < 0.5 and over <= max(1, 0.05 * sure.numel()) and float(err.median()) < 0.03, (worst, over, float(err.median()))
+
+
+def portions(n, sizes):
+    out, i, k = [], 0, 0
+    while i < n:
+        s = min(sizes[k % len(sizes)], n - i)
+        out.append(s)
+        i += s
+        k += 1
+    return out
+
+
+def replay_alone(eng, rid, toks, cuts):
+    """Feed `toks` in the given portion sizes; logits of every position."""
+    rows, i = [], 0
+    for c in cuts:
+        rows.append(eng.replay_step([(rid, toks[i:i + c], list(range(c)))], [rid] if i + c == len(toks) else []))
+        i += c
+    return torch.cat(rows, 0)
+
+
+def rand_tokens(cfg, n, seed):
+    return np.random.default_rng(seed).integers(0, cfg["vocab"], size=n).tolist()
+
+
+_ORACLE = {}
+
+
+def fwd(cfg, W, toks, streams=None):
+    """The oracle on one sequence (kept per configuration and token list: several tests ask for the same)."""
+    if streams is not None:
+        return oracle.forward(cfg, W, toks, streams=streams)
+    key = (json.dumps(cfg, sort_keys=True), tuple(toks))
+    if key not in _ORACLE:
+        margins = [float("inf")] * len(toks)
+        _ORACLE[key] = Want(oracle.forward(cfg, W, toks, margins=margins), margins)
+    return _ORACLE[key]
+
+
+def on_cpu_only_in_fp32(name, device, dtype):
+    """The configuration made for the GPU's specialised paths is slow in the plain oracle: the CPU runs it once."""
+    if name == "wide" and device == "cpu" and dtype != "float32":
+        pytest.skip("the wide configuration runs on the CPU in fp32 only")
+
+
+# --------------------------------------------------------------------------------------- whole prompts
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("name", ["small", "varied", "tail", "odd", "wide"])
+def test_whole_prompt_matches_oracle(ckpt, name, device, dtype):
+    on_cpu_only_in_fp32(name, device, dtype)
+    path, cfg, W = ckpt(name)
+    toks = rand_tokens(cfg, 60, 1)            # past most windows, pages of 16
+    want = fwd(cfg, W, toks)
+    eng = engine(path, device, dtype)
+    close(replay_alone(eng, 1, toks, [len(toks)]), want, dtype)
+    # the very first tokens: a one-token prompt, then two (zero state, zeros before the convolution, a sink and one key)
+    close(replay_alone(eng, 2, toks[:1], [1]), fwd(cfg, W, toks[:1]).logits, dtype)
+    close(replay_alone(eng, 3, toks[:2], [2]), want[:2], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", ["varied", "small", "wide"])
+def test_residual_stream_after_every_layer_run(ckpt, name, device):
+    if name == "wide" and device == "cpu":
+        pytest.skip("the wide configuration's streams are compared on the GPU")
+    path, cfg, W = ckpt(name)
+    toks = rand_tokens(cfg, 23, 2)
+    want = []
+    fwd(cfg, W, toks, want)
+    eng = engine(path, device, "float32")
+    got = []
+    from localai_amd.models.decoder import ForwardBatch
+    eng.sched.add(1, toks, 0)
+    plan = eng.sched.schedule_explicit([(1, len(toks))])
+    fb = ForwardBatch(tokens=eng._dev(plan["p_tokens"]), pos=eng._dev(plan["p_pos"]), slots=eng._dev(plan["p_slots"]),
+                      decode=False, block_tables=eng._dev(plan["p_bt"]), cu_q=eng._dev(plan["p_cu"]),
+                      ctx_lens=eng._dev(plan["p_ctx"]), sslots=eng._dev(plan["p_sslot"]),
+                      row_seq=eng._dev(np.zeros(len(toks), dtype=np.int32)))
+    eng.model.forward(fb, eng.kv, layer_out=got)
+    assert len(got) == len(want) == len(oracle.runs(cfg)) == len(eng.kv.k)
+    for a, b in zip(got, want):
+        assert float((a.cpu() - b).abs().max()) < 2e-4 * max(1.0, float(b.abs().max()))
+
+
+# --------------------------------------------------------------------------------------- portions, decoding
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("name", ["varied", "tail", "odd", "wide"])
+def test_portions_and_token_by_token_decoding(ckpt, name, device, dtype):
+    if name == "wide" and device == "cpu":
+        pytest.skip("the wide configuration's portions run on the GPU")
+    path, cfg, W = ckpt(name)
+    toks = rand_tokens(cfg, 60, 3)
+    want = fwd(cfg, W, toks)
+    eng = engine(path, device, dtype)
+    for rid, cuts in enumerate([portions(60, [2]), portions(60, [5, 2, 17, 3, 31]), portions(60, [34, 1, 1, 7]),
+                                [25] + [1] * 35, [1] * 60], 1):
+        close(replay_alone(eng, rid, toks, cuts), want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+def test_long_decoding_over_windows_and_pages(ckpt, device, dtype):
+    path, cfg, W = ckpt("small")
+    toks = rand_tokens(cfg, 110, 4)           # windows 9 and 12, pages of 16, two passes of the looped layers
+    want = fwd(cfg, W, toks)
+    eng = engine(path, device, dtype)
+    close(replay_alone(eng, 1, toks, [10] + [1] * 100), want, dtype)
+
+
+# --------------------------------------------------------------------------------------- batches, reuse
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("name", ["small", "wide"])
+def test_mixed_batches_of_unequal_requests_with_page_and_slot_reuse(ckpt, name, device, dtype):
+    """Four live requests at most in a pool of 160 tokens with 4 state slots, ten requests in all:
+    portions of some beside single tokens of others, every finished request's pages and slot taken
+    over by the next (whose convolution tail, memories and running maximum must start from zero,
+    not from the leftovers).  Every position must equal the request run alone (the oracle)."""
+    if name == "wide" and device == "cpu":
+        pytest.skip("the wide configuration's batches run on the GPU")
+    path, cfg, W = ckpt(name)
+    rng = np.random.default_rng(5)
+    lens = [33, 7, 48, 2, 21, 40, 1, 17, 30, 9]
+    reqs = {i + 1: rand_tokens(cfg, n, 100 + i) for i, n in enumerate(lens)}
+    want = {i: fwd(cfg, W, t) for i, t in reqs.items()}
+    eng = engine(path, device, dtype, tokens=160, slots=4, bs=16)
+    pending = list(reqs)
+    live, at = [], {}
+    got = {i: [] for i in reqs}
+    while pending or live:
+        while pending and len(live) < 4 and sum(-(-len(reqs[i]) // 16) * 16 for i in live + pending[:1]) <= 160:
+            live.append(pending.pop(0))
+            at[live[-1]] = 0
+        entries = []
+        for i in live:
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                       # rests this step
+            left = len(reqs[i]) - at[i]
+            n = min(left, int(rng.choice([1, 1, 2, 3, 8, 19])))
+            entries.append((i, reqs[i][at[i]:at[i] + n], list(range(n))))
+        if not entries:
+            continue
+        end = [i for i, t, _ in entries if at[i] + len(t) == len(reqs[i])]
+        lg = eng.replay_step(entries, end)
+        o = 0
+        for i, t, _ in entries:
+            got[i].append(lg[o:o + len(t)])
+            o += len(t)
+            at[i] += len(t)
+        for i in end:
+            live.remove(i)
+    assert eng.sched.num_free_state_slots == 4 and eng.sched.blocks().num_free == 10
+    for i in reqs:
+        close(torch.cat(got[i], 0), want[i], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_pools_follow_the_layer_runs(ckpt, device):
+    """One entry per layer RUN (a looped layer once per pass): a delta layer holds a convolution tail
+    (serving dtype) and an fp32 state, a latent layer one-head pages of rank + rot_dim and no V pages,
+    a parallel layer K / V pages plus the memory (with its normaliser column) and the running maximum."""
+    path, cfg, W = ckpt("small")
+    eng = engine(path, device, "bfloat16", tokens=64, slots=2, bs=16)
+    kv = eng.kv
+    assert len(kv.k) == len(kv.state) == 6          # 0, (1, 2), (1, 2), 3
+    assert kv.k[0] is None and kv.k[5] is None
+    tail, state = kv.state[0]
+    assert tail.dtype == torch.bfloat16 and tuple(tail.shape) == (2, 2, 2 * 2 * 8 + 4 * 6)
+    assert state.dtype == torch.float32 and tuple(state.shape) == (2, 4, 6, 8)
+    for r in (1, 3):
+        assert tuple(kv.k[r].shape[1:]) == (1, 16, 14) and kv.v[r] is None and kv.state[r] is None
+    for r in (2, 4):
+        assert tuple(kv.k[r].shape[1:]) == (2, 16, 12) and tuple(kv.v[r].shape[1:]) == (2, 2, 8, 8)
+        mem, mx = kv.state[r]
+        assert mem.dtype == mx.dtype == torch.float32 and tuple(mem.shape) == (2, 2, 11, 6) and tuple(mx.shape) == (2, 2)
+    assert kv.k[1].data_ptr() != kv.k[3].data_ptr()     # every pass has pages of its own
+    assert eng.model.kv_bytes_per_token() == 2 * 2 * (14 + 2 * (12 + 8))
+
+
+# --------------------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("device,dtype,graphs,name", [
+    ("cpu", "float32", False, "small"),
+    pytest.param("cuda:0", "float32", False, "small", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "bfloat16", True, "small", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "float32", True, "varied", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "bfloat16", True, "wide", marks=pytest.mark.gpu),
+    pytest.param("cuda:0", "bfloat16", False, "wide", marks=pytest.mark.gpu)])
+def test_greedy_generation_through_the_engine(ckpt, device, dtype, graphs, name):
+    """engine.add_request / step: scheduler-planned chunked prefill, (graph-replayed multi-step)
+    decode with the device sampler, several requests at once; every emitted token is the oracle's
+    argmax at its position unless the oracle's top-2 margin is within rounding."""
+    path, cfg, W = ckpt(name)
+    eng = LLMEngine(EngineConfig(model_path=path, device=device, context_size=128, max_num_seqs=4,
+                                 max_batched_tokens=24, block_size=16, use_graphs=graphs, dtype=dtype,
+                                 record_tokens=True, decode_steps=4, decode_steps_wide=4))
+    prompts = [rand_tokens(cfg, n, 200 + n) for n in (5, 30, 47)]
+    done = {}
+    for k, p in enumerate(prompts):
+        def cb(ev, k=k):
+            if ev.finished:
+                done[k] = ev
+        eng.add_request(p, SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True), cb)
+    for _ in range(400):
+        if len(done) == len(prompts):
+            break
+        eng.step()
+    assert len(done) == len(prompts)
+    margin_ok = 1e-3 if dtype == "float32" else 0.1
+    for k, p in enumerate(prompts):
+        gen = done[k].token_ids
+        assert len(gen) == 20
+        ref = fwd(cfg, W, p + gen[:-1])
+        for j, t in enumerate(gen):
+            row = ref.logits[len(p) - 1 + j]
+            top2 = torch.topk(row, 2).values
+            if dtype != "float32" and float(ref.margins[:len(p) + j].min()) < MARGIN:
+                break       # a close router call upstream: from here on the oracle may follow other experts
+            assert t == int(row.argmax()) or float(top2[0] - top2[1]) <= margin_ok, (k, j)
+    assert eng.sched.num_free_state_slots == 4
+
+
+def test_registry_reader_and_configuration(ckpt):
+    from localai_amd.models import model_class
+    from localai_amd.models.gosuvik import GosuvikModel
+    from localai_amd.models.hf_checkpoint import open_model
+    path, cfg, W = ckpt("varied")
+    r = open_model(path)
+    assert r.architecture == "gosuvik" and model_class(r.architecture) is GosuvikModel
+    m = GosuvikModel(r, torch.device("cpu"), dtype=torch.float32)
+    hp = m.hp
+    assert [x.kind for x in hp.mixers] == ["parallel", "latent_attention", "channel_delta", "latent_attention", "parallel"]
+    assert hp.loop is None and hp.runs == [0, 1, 2, 3, 4] and hp.norm_groups == 1 and hp.mlps[1] is None
+    assert (hp.mixers[0].left.window, hp.mixers[0].left.rot.scaling, hp.mixers[0].right.gate_cap) == (40, None, 15.0)
+    assert (hp.mixers[1].window, hp.mixers[1].rot.scaling, hp.mixers[3].rot.scaling["original"]) == (0, None, 16)
+    assert (hp.mixers[2].taps, hp.mixers[2].kv_heads, m.layers[2].rank_a, m.layers[2].rank_g) == (1, 3, 3, 2)
+    assert (hp.mlps[3].experts, hp.mlps[3].top, hp.mlps[0].top) == (7, 4, 3)
+    assert (hp.mixers[4].left_scale, hp.mixers[4].right_scale) == (0.3, 1.5)
+    # linear scaling divides every frequency; YaRN leaves the fast ones and sets a magnitude
+    f = m.layers[4].freqs.cpu()
+    assert torch.allclose(f, torch.tensor([50.0 ** (-2.0 * i / 6) / 8.0 for i in range(3)]), rtol=1e-6) and m.layers[4].mag == 1.0
+    assert m.layers[3].mag == pytest.approx(0.1 * np.log(2.0) + 1.0)
+    looped = type(hp).from_config(CONFIGS["tail"])
+    assert looped.runs == [0, 1, 2] * 3 and type(hp).from_config(CONFIGS["odd"]).runs == [0, 1, 2, 2]
+    bad = dict(cfg, layers=[dict(cfg["layers"][0], type="convolution")])
+    with pytest.raises(ValueError):
+        type(hp).from_config(bad)
+    with pytest.raises(ValueError):
+        type(hp).from_config(dict(cfg, loop={"start": 2, "stop": 9, "times": 2}))
+
+
+def test_trace_runner_cli(ckpt, tmp_path):
+    """The schedule replay program end to end on the CPU: two requests, a rest, a reused name."""
+    import subprocess
+    import sys
+    path, cfg, W = ckpt("tail")
+    a, b = rand_tokens(cfg, 20, 7), rand_tokens(cfg, 9, 8)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[11:13], "want": []}, {"id": "b", "tokens": b, "want": [8]}],
+              "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[13:], "want": [6]}, {"id": "b", "tokens": a[:3], "want": [2]}],
+              "end": ["a", "b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "64", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    wa, wb = fwd(cfg, W, a), fwd(cfg, W, b)
+    V = cfg["vocab"]
+    g = [torch.from_numpy(np.fromfile(out / f"{k}.f32", dtype="<f4").reshape(-1, V)) for k in range(3)]
+    close(g[0], wa.logits[[0, 10]], "float32")
+    close(g[1], wb.logits[[8]], "float32")
+    close(g[2], torch.stack([wa.logits[19], wa.logits[2]]), "float32")
+
+
+def test_backend_service_loads_and_generates(ckpt, monkeypatch):
+    """The gRPC backend servicer (what the gateway talks to): LoadModel on the checkpoint directory,
+    Predict with a numeric prompt; greedy tokens follow the oracle."""
+    import asyncio
+    from localai_amd.grpc import backend_pb as pb
+    from localai_amd.grpc.servicer import EngineServicer
+    monkeypatch.setenv("LOCALAI_MAX_NUM_SEQS", "4")
+    path, cfg, W = ckpt("tail")
+    prompt = [3, 17, 5, 9, 30]
+
+    async def run():
+        sv = EngineServicer(device="cpu")
+        r = await sv.LoadModel(pb.ModelOptions(ModelFile=path, ContextSize=64))
+        assert r.success, r.message
+        return await sv.Predict(pb.PredictOptions(Prompt=" ".join(str(t) for t in prompt), Tokens=5, Temperature=0.0,
+                                                  IgnoreEOS=True))
+    rep = asyncio.run(run())
+    gen = [int(x) for x in rep.message.decode().strip("<>").split("><")]
+    assert rep.tokens == 5 and rep.prompt_tokens == len(prompt) and len(gen) == 5
+    ref = fwd(cfg, W, prompt + gen[:-1])
+    for j, t in enumerate(gen):
+        row = ref.logits[len(prompt) - 1 + j]
+        top2 = torch.topk(row, 2).values
+        if float(ref.margins[:len(prompt) + j].min()) < MARGIN:
+            break
+        assert t == int(row.argmax()) or float(top2[0] - top2[1]) <= 0.1, j      # served in bf16 by default
