@@ -228,7 +228,8 @@ def close(got, want, dtype):
         sure = err if margins is None else err[margins > MARGIN]
         worst = float(sure.max()) if sure.numel() else 0.0
         over = int((sure > 0.12).sum())       # 16-bit rounding ahead of a sharp gate or softmax: a few positions stand out
-        assert worst < 0.5 and over <= max(1, 0.05 * sure.numel()) and float(err.median()) < 0.03, (worst, over, float(err.median()))
+        med = 0.03 if err.numel() >= 8 else 0.08          # a request of a token or two has no median to speak of
+        assert worst < 0.5 and over <= max(1, 0.05 * sure.numel()) and float(err.median()) < med, (worst, over, float(err.median()))
 
 
 def portions(n, sizes):

@@ -1,0 +1,342 @@
+"""Gosuvik's mechanisms one at a time against the plain oracle of tests/gosuvik_oracle.py: the new
+operators directly, and every mixer and feed-forward alone through the model's own methods with
+hand-made batches (portions, pages in any order, decode rows, slots taken over), on inputs made so
+that a fault shows: a row that towers over the others just inside and just outside a window, far
+back, at a page border; sinks that swallow a head or vanish; gates driven to both ends.
+"""
+import numpy as np
+import pytest
+import torch
+
+import gosuvik_oracle as oracle
+from localai_amd import ops
+from localai_amd.models.decoder import ForwardBatch
+from localai_amd.models.gosuvik import GosuvikModel
+from localai_amd.models.hf_checkpoint import open_model
+from test_gosuvik import delta, dense, latent, make_weights, moe, parallel, write_checkpoint, clean
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+MODES = [("cpu", "float32"), pytest.param("cuda:0", "float32", marks=pytest.mark.gpu),
+         pytest.param("cuda:0", "bfloat16", marks=pytest.mark.gpu)]
+F64 = torch.float64
+
+
+def rel(got, want):
+    got, want = got.detach().double().cpu(), want.double()
+    return float((got - want).norm() / want.norm().clamp_min(1e-12))
+
+
+def tol(dtype):
+    return 2e-5 if dtype in ("float32", torch.float32) else 2e-2
+
+
+# ------------------------------------------------------------------------------------------- operators
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("D,groups", [(48, 4), (36, 3), (40, 1), (35, 5), (256, 8), (2048, 2), (4100, 4), (96, 96)])
+def test_group_norm_boundary(device, D, groups):
+    g = torch.Generator().manual_seed(D)
+    T = 5
+    res0 = torch.randn(T, D, generator=g) * 3
+    w = 1 + 0.3 * torch.randn(D, generator=g)
+    for kind in ("none", "f32", "bf16", "slabs"):
+        res = res0.clone().to(device)
+        if kind == "none":
+            br, add = None, 0
+        elif kind == "slabs":
+            sl = torch.randn(3, T, D, generator=g)
+            br, add = ops.Partial(sl.to(device)), sl.sum(0)
+        else:
+            b = torch.randn(T, D, generator=g).to(torch.float32 if kind == "f32" else torch.bfloat16)
+            br, add = b.to(device), b.float()
+        out = ops.add_group_norm(res, br, w.to(device), 1e-5, groups, out_dtype=torch.float32)
+        want = oracle.group_norm((res0 + add).to(F64), w.to(F64), 1e-5, groups)
+        assert rel(out, want) < 2e-6 and rel(res, res0 + add) < 1e-6
+        out16 = ops.add_group_norm(res0.clone().to(device), br, w.to(device), 1e-5, groups)
+        assert out16.dtype == torch.bfloat16 and rel(out16, want) < 5e-3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("F", [13, 256, 1000])
+def test_polynomial_activation(device, F):
+    g = torch.Generator().manual_seed(F)
+    z = (torch.randn(6, F, generator=g) * 2).to(torch.bfloat16)
+    z[3] = z[3] * 0.01       # a row whose powers vanish beside eps
+    for coef in ([0.7, -0.4, 0.2, 0.1], [0.0, 1.0, 0.0, 0.0], [0.0, 0.0, 0.0, -2.0]):
+        c = torch.tensor(coef)
+        zf = z.to(F64)
+        want = sum(coef[k] * oracle.unit_rms(zf ** (k + 1), 1e-5) for k in range(3)) + coef[3]
+        for src in (z.to(device), z.float().to(device), ops.Partial(torch.stack([z.float() * 0.25, z.float() * 0.75]).to(device))):
+            out = ops.poly_norm_act(src, c.to(device), 1e-5, out_dtype=torch.float32)
+            assert rel(out, want) < 3e-6
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_sigmoid_gate_reads_columns_of_a_wider_row(device):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(7, 30, generator=g)
+    wide = torch.randn(7, 75, generator=g) * 4
+    for dt in (torch.float32, torch.bfloat16):
+        xd, wd = x.to(dt).to(device), wide.to(dt).to(device)
+        out = ops.sigmoid_mul(xd, wd[:, 21:51], out_dtype=torch.float32)
+        want = xd.cpu().to(F64) * oracle.sigmoid(wd.cpu()[:, 21:51].to(F64))
+        assert rel(out, want) < 2e-6
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("H,G,D,Dv,rot", [(4, 2, 12, 8, 8), (3, 1, 10, 14, 2), (2, 2, 64, 64, 64), (6, 3, 16, 6, 0)])
+def test_normed_rotated_pages_and_turn_back(device, H, G, D, Dv, rot):
+    """q / k norms with weights, partial rotation with scaled positions, values rotated over their
+    whole width into the pages (with leftovers in the pool, a row without a slot), and rotate_heads
+    taking them back: rotating a cached value by minus its position gives the plain value."""
+    g = torch.Generator().manual_seed(H * 100 + D)
+    T, BS = 9, 8
+    src = torch.randn(T, (H + G) * D + G * Dv + 5, generator=g)      # columns to spare: a wider projection
+    qw, kw = 1 + 0.3 * torch.randn(D, generator=g), 1 + 0.3 * torch.randn(D, generator=g)
+    pos = torch.tensor([0, 1, 2, 3, 40, 41, 1000, 7, 8], dtype=torch.int32)
+    slots = torch.tensor([16, 17, 18, 19, 0, 1, 9, -1, 31], dtype=torch.int32)
+    freqs, mag = oracle.rot_table(rot, 50.0, {"factor": 4.0}) if rot else ([], 1.0)
+    vfreqs, _ = oracle.rot_table(Dv, 50.0)
+    fq = ops.linear_rot_freqs(rot, 50.0, 4.0, device)
+    fv = ops.linear_rot_freqs(Dv, 50.0, 1.0, device)
+    assert rel(fv, torch.tensor(vfreqs)) < 1e-6
+    kc = torch.full((4, G, BS, D), 7.0).to(device)
+    vc = torch.full((4, G, BS // 8, Dv, 8), 7.0).to(device)
+    q = ops.qk_norm_rope_pages(src.to(device), H, D, G, Dv, pos.to(device), slots.to(device), qw.to(device), kw.to(device),
+                               1e-5, fq, 1.0, rot, fv, kc, vc)
+    s64 = src.to(F64)
+    for t in range(T):
+        qq = oracle.rotate_halves(oracle.unit_rms(s64[t, :H * D].view(H, D), 1e-5) * qw.to(F64), int(pos[t]), freqs, mag)
+        assert rel(q[t].view(H, D), qq) < 5e-5       # fp32 angles: position 1000 rounds at 6e-5 rad
+        if slots[t] < 0:
+            continue
+        b, o = int(slots[t]) // BS, int(slots[t]) % BS
+        kk = oracle.rotate_halves(oracle.unit_rms(s64[t, H * D:(H + G) * D].view(G, D), 1e-5) * kw.to(F64), int(pos[t]), freqs, mag)
+        v0 = s64[t, (H + G) * D:(H + G) * D + G * Dv].view(G, Dv)
+        assert rel(kc[b, :, o], kk) < 5e-5
+        assert rel(vc[b, :, o // 8, :, o % 8], oracle.rotate_halves(v0, int(pos[t]), vfreqs)) < 5e-5
+    assert float(kc[1, :, 2:].min()) == 7.0 and float(kc[3, :, :7].min()) == 7.0      # nothing else was touched
+    # the turn-back, into a window of a wider buffer, with a scale
+    x = torch.randn(T, H * Dv, generator=g)
+    buf = torch.full((T, H * Dv + 6), 3.0).to(device)
+    ops.rotate_heads(x.to(device), H, Dv, pos.to(device), fv, -1.0, 0.6, out=buf, col0=4)
+    for t in range(T):
+        want = 0.6 * oracle.rotate_halves(x[t].to(F64).view(H, Dv), -int(pos[t]), vfreqs)
+        assert rel(buf[t, 4:4 + H * Dv].view(H, Dv), want) < 5e-5
+    assert float(buf[:, :4].min()) == 3.0 and float(buf[:, 4 + H * Dv:].max()) == 3.0
+
+
+# ------------------------------------------------------------------------------------------- mixers alone
+def build(layer, D, tmp_path, device, dtype, seed=0, edit=None):
+    """A one-layer checkpoint and its model: (model, config of the layer's mixer, float weights)."""
+    cfg = {"vocab": 11, "width": D, "norm": {"eps": 1e-5, "groups": 1}, "layers": [layer]}
+    W = make_weights(cfg, seed)
+    if edit:
+        edit(W)
+    path = str(tmp_path / f"m{seed}_{device.replace(':', '')}_{dtype}")
+    write_checkpoint(path, cfg, W)
+    m = GosuvikModel(open_model(path), torch.device(device), dtype=getattr(torch, dtype))
+    return m, clean(cfg)["layers"][0], {k: v.float() for k, v in W.items()}
+
+
+class Seq:
+    """One sequence's pages (in the order given) and state slot in a pool."""
+
+    def __init__(self, table, slot):
+        self.table, self.slot, self.at = list(table), slot, 0
+
+
+def run_mixer(model, kv, seq, h, cuts, bs, decode_rows=True):
+    """Feed rows h (the mixer's input) of one sequence in portions through layer 0's mixer and output
+    projection; single rows as decode batches when decode_rows.  fp32 [T, D]."""
+    dev, L, m = model.device, model.layers[0], model.hp.mixers[0]
+    outs, i = [], 0
+    tab = torch.tensor([seq.table], dtype=torch.int32, device=dev)
+    for c in cuts:
+        p0 = seq.at
+        pos = torch.arange(p0, p0 + c, dtype=torch.int32)
+        slots = torch.tensor([seq.table[p // bs] * bs + p % bs for p in pos.tolist()], dtype=torch.int32)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)  # noqa: E731
+        dec = decode_rows and c == 1 and p0 > 0
+        fb = ForwardBatch(tokens=i32([0] * c), pos=pos.to(dev), slots=slots.to(dev), decode=dec, block_tables=tab,
+                          sslots=i32([seq.slot]))
+        if dec:
+            fb.seq_lens, fb.max_len = i32([p0 + 1]), p0 + 1
+            row_seq, cu_q, tiles = model._single_rows(1)
+            tile_rows = 1 if (not model.f32 and dev.type == "cuda") else 0
+            splits = 2
+        else:
+            fb.cu_q, fb.ctx_lens, fb.row_seq, fb.max_q = i32([0, c]), i32([p0 + c]), i32([0] * c), c
+            tiles, tile_rows = model.prefill_tiles([c], dev)
+            row_seq, cu_q, splits = fb.row_seq, fb.cu_q, 1
+        xn = h[i:i + c].to(model.dtype).to(dev).contiguous()
+        if m.kind == "channel_delta":
+            a = model._delta(L, m, xn, fb, kv, 0, cu_q)
+        elif m.kind == "latent_attention":
+            a = model._latent(L, m, xn, fb, kv, 0, row_seq, splits)
+        else:
+            a = model._parallel(L, m, xn, fb, kv, 0, row_seq, cu_q, tiles, tile_rows, splits, None)
+        outs.append(model._dense(ops.linear(a, L.wo)).float().cpu())
+        seq.at += c
+        i += c
+    return torch.cat(outs, 0)
+
+
+def inputs(T, D, seed, hot=()):
+    """Normed-looking rows; the rows listed in `hot` tower over the others (a key, value or write that
+    cannot be missed, nor seen by mistake)."""
+    g = torch.Generator().manual_seed(seed)
+    h = torch.randn(T, D, generator=g).to(torch.bfloat16).float()
+    for t in hot:
+        h[t] = h[t] * 12
+    return h
+
+
+ORACLE = {"channel_delta": oracle.channel_delta, "latent_attention": oracle.latent_attention, "parallel": oracle.parallel}
+
+
+def check_mixer(model, layer, W, h, cuts_list, bs, nblocks, dtype, tables=None):
+    want = ORACLE[layer["type"]](({k: v.to(F64) for k, v in W.items()}), "l0.mix.", layer["mixer"], h.to(F64), 1e-5)
+    kv = model.new_kv_cache(nblocks, bs, state_slots=3)
+    T = h.shape[0]
+    need = -(-T // bs)
+    for n, cuts in enumerate(cuts_list):
+        # pages in another order every time, slots in turn: leftovers of the run before lie in both
+        table = (tables[n] if tables else list(np.random.default_rng(n).permutation(nblocks)[:need]))
+        got = run_mixer(model, kv, Seq(table, n % 3), h, cuts, bs)
+        err = ((got.double() - want).norm(dim=-1) / want.norm(dim=-1).clamp_min(1e-9))
+        assert float(err.max()) < (1e-4 if dtype == "float32" else 6e-2), (n, int(err.argmax()), float(err.max()))
+
+
+def cuts_of(T, *sizes):
+    out, i, k = [], 0, 0
+    while i < T:
+        s = min(sizes[k % len(sizes)], T - i)
+        out.append(s)
+        i += s
+        k += 1
+    return out
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("spec", [dict(heads=4, kv=2, dim=8, vdim=6, conv=3), dict(heads=3, kv=3, dim=5, vdim=7, conv=1),
+                                  dict(heads=2, kv=1, dim=64, vdim=64, conv=4), dict(heads=2, kv=2, dim=40, vdim=72, conv=5),
+                                  dict(heads=1, kv=1, dim=200, vdim=16, conv=2)])
+def test_delta_rule_alone(tmp_path, device, dtype, spec):
+    """Whole, in portions down to two rows and one, token by token; the first rows of a sequence (zeros
+    before the convolution, zero state), hot rows whose write every later read-out sees."""
+    model, layer, W = build(dense(delta(**spec), 0), 32, tmp_path, device, dtype)
+    T = 45
+    h = inputs(T, 32, 1, hot=(0, 17))
+    check_mixer(model, layer, W, h, [[T], cuts_of(T, 2), cuts_of(T, 1), cuts_of(T, 7, 1, 2, 16), [30] + [1] * 15], 16, 6, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+def test_delta_rule_forgets_and_keeps(tmp_path, device, dtype):
+    """Decays driven to both ends: channels that forget at once and channels that keep everything over
+    300 rows, write strengths at 0 and 1; the state of a slot is taken over from another sequence."""
+    def edit(W):
+        W["l0.mix.dt_bias"][:8] = -30.0          # softplus -> 0: these key channels never decay
+        W["l0.mix.dt_bias"][8:16] = 12.0         # ... and these forget within a row
+        W["l0.mix.b"][0] = W["l0.mix.b"][0] * 40     # beta at 0 or 1
+    model, layer, W = build(dense(delta(heads=2, kv=1, dim=16, vdim=8, conv=3), 0), 24, tmp_path, device, dtype, edit=edit)
+    T = 300
+    h = inputs(T, 24, 2, hot=(3,))
+    check_mixer(model, layer, W, h, [[T], [150] + [1] * 150, cuts_of(T, 33, 2)], 16, 20, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("spec", [dict(heads=3, dim=8, rot_dim=4, vdim=6, rank=10, window=12),
+                                  dict(heads=2, dim=5, rot_dim=6, vdim=7, rank=9, window=0, scaling=None),
+                                  dict(heads=4, dim=32, rot_dim=32, vdim=48, rank=96, window=21, base=10000.0, scale=0.12),
+                                  dict(heads=16, dim=16, rot_dim=16, vdim=16, rank=48, window=33, scale=0.2),
+                                  dict(heads=2, dim=24, rot_dim=8, vdim=40, rank=56, window=64, scale=0.2)])
+def test_latent_attention_alone(tmp_path, device, dtype, spec):
+    """Hot rows placed so that queries see them at the window's last place and miss them one later, in
+    a portion and decoded alone, at a page border (pages of 16) and far back (no window)."""
+    model, layer, W = build(dense(latent(**spec), 0), 32, tmp_path, device, dtype)
+    w = spec["window"] or 1000
+    T = 100
+    h = inputs(T, 32, 3, hot=(0, 15, 16, 50))
+    cuts = [[T], cuts_of(T, 2), [15 + w - 1, 1, 1, 1] + cuts_of(T - 15 - w - 2, 9, 1) if 15 + w + 2 < T else cuts_of(T, 31, 1),
+            [40] + [1] * 60]
+    check_mixer(model, layer, W, h, cuts, 16, 8, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("spec", [dict(), dict(heads=3, kv=1, dim=10, vdim=14, rot=2, window=33, factor=3.0, r_heads=3, r_dim=7, r_vdim=9),
+                                  dict(heads=4, kv=2, dim=64, vdim=32, rot=32, window=24, scale=0.125, r_heads=2, r_dim=64, r_vdim=64),
+                                  dict(heads=8, kv=2, dim=64, vdim=64, rot=64, window=17, factor=2.0, scale=0.125, r_heads=4,
+                                       r_dim=32, r_vdim=96, cap=10.0),
+                                  dict(heads=2, kv=2, dim=32, vdim=16, rot=16, window=0, factor=0, r_heads=1, r_dim=130, r_vdim=20,
+                                       cap=3.0, ls=1.0, rs=1.0)])
+def test_parallel_mixer_alone(tmp_path, device, dtype, spec):
+    """Sink attention with rotated values beside the matrix memory: hot rows at the window's edge, at
+    page borders, far back; portions, decode rows (the split-KV decode kernel where the widths allow)."""
+    model, layer, W = build(dense(parallel(**spec), 0), 32, tmp_path, device, dtype)
+    w = layer["mixer"]["left"].get("mask", {}).get("size", 1000)
+    T = 100
+    h = inputs(T, 32, 4, hot=(0, 15, 16, 47))
+    cuts = [[T], cuts_of(T, 2), [15 + w - 1, 1, 1, 1] + cuts_of(T - 15 - w - 2, 9, 1) if 15 + w + 2 < T else cuts_of(T, 31, 1),
+            [40] + [1] * 60]
+    check_mixer(model, layer, W, h, cuts, 16, 8, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("sink", [30.0, -30.0])
+def test_sink_swallows_a_head_or_vanishes(tmp_path, device, dtype, sink):
+    def edit(W):
+        W["l0.mix.left.sink"][0] = sink
+        W["l0.mix.left.sink"][1] = -sink
+    model, layer, W = build(dense(parallel(heads=4, kv=2, dim=32, vdim=16, rot=16, window=20, rs=0.0), 0), 32, tmp_path, device,
+                            dtype, edit=edit)
+    h = inputs(50, 32, 5)
+    check_mixer(model, layer, W, h, [[50], [20] + [1] * 30], 16, 4, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+def test_matrix_memory_gates_at_both_ends_and_long_rows(tmp_path, device, dtype):
+    """Input gates far above and forget gates far below the running maximum, a head that keeps
+    everything; 1100 rows in one portion (scanned in segments on the GPU), then continued in portions
+    and single rows from the slot; the attention branch is switched off by its scale."""
+    def edit(W):
+        W["l0.mix.right.f.b"][0] = 9.0           # forget gate ~ 1: nothing decays, m follows the inputs
+        W["l0.mix.right.f.b"][1] = -6.0          # ... and one that forgets fast
+        W["l0.mix.right.i.b"][2] = 6.0
+    model, layer, W = build(dense(parallel(heads=2, kv=1, dim=8, vdim=8, rot=4, window=8, ls=0.0, rs=1.0, r_heads=4, r_dim=24,
+                                           r_vdim=64, cap=9.0), 0), 40, tmp_path, device, dtype, edit=edit)
+    T = 1160
+    h = inputs(T, 40, 6, hot=(0, 500))
+    check_mixer(model, layer, W, h, [[1100, 30, 2, 1, 1] + [13, 13], [T]], 16, 80, dtype,
+                tables=[list(range(73)), list(range(79, 6, -1))])
+
+
+# ------------------------------------------------------------------------------------------- feed-forwards
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("experts,top,n,T", [(5, 2, 24, 9), (3, 3, 10, 40), (6, 1, 18, 70), (70, 6, 8, 5)])
+def test_routed_experts_alone(tmp_path, device, dtype, experts, top, n, T):
+    model, layer, W = build(moe(delta(), experts=experts, top=top, n=n), 32, tmp_path, device, dtype)
+    h = inputs(T, 32, 7)
+    W64 = {k: v.to(F64) for k, v in W.items()}
+    ids, w, margin = oracle.router(W64, "l0.mlp.", layer["mlp"], h.to(F64))
+    want = oracle.expert_ff(W64, "l0.mlp.", layer["mlp"], h.to(F64))
+    got = model._mlp(model.layers[0], model.hp.mlps[0], h.to(model.dtype).to(model.device))
+    got = (got.dense() if isinstance(got, ops.Partial) else got).float().cpu()
+    sure = margin > (1e-4 if dtype == "float32" else 0.1)
+    assert int(sure.sum()) >= T // 3
+    assert rel(got[sure], want[sure]) < (1e-5 if dtype == "float32" else 3e-2)
+    gi, gw = ops.router_softmax(h.to(model.device), model.layers[0].router, None, top)
+    for t in range(T):
+        if sure[t]:
+            assert sorted(gi[t].tolist()) == sorted(ids[t].tolist())
+            order = torch.argsort(gi[t].cpu())
+            assert rel(gw.view(T, top)[t].cpu()[order], w[t][torch.argsort(ids[t])]) < 1e-5
+
+
+@pytest.mark.parametrize("device,dtype", MODES)
+@pytest.mark.parametrize("ff", [13, 40, 512])
+def test_polynomial_feed_forward_alone(tmp_path, device, dtype, ff):
+    model, layer, W = build(dense(delta(), ff), 32, tmp_path, device, dtype)
+    h = inputs(12, 32, 8)
+    want = oracle.poly_ff({k: v.to(F64) for k, v in W.items()}, "l0.mlp.", h.to(F64), 1e-5)
+    got = model._mlp(model.layers[0], model.hp.mlps[0], h.to(model.dtype).to(model.device))
+    assert rel(model._dense(got).float().cpu(), want) < (1e-5 if dtype == "float32" else 3e-2)
