@@ -78,7 +78,7 @@ def parse():
                          "other ranks' engines answer it over backend.proto gRPC")
     ap.add_argument("--design-compare", default="",
                     help="instead of the headline workload: prefill and decode tokens/s of a model design "
-                         "(suganex, dadizen, vinozen) beside the closest decoder family at equal layer sizes, random weights, one GPU")
+                         "(suganex, dadizen, vinozen, gosuvik) beside the closest decoder family at equal layer sizes, random weights, one GPU")
     ap.add_argument("--design-sizes", default="2k,4k", help="--design-compare: layer sizes (2k, 4k)")
     ap.add_argument("--n-draft", type=int, default=0,
                     help="engine mode: n-gram speculative draft length (model-config n_draft); 0 = off")

@@ -1510,3 +1510,86 @@ def write_vinozen(out_dir: str, width: int = 256, kinds=("attention", "mamba2"),
         json.dump(cfg, f_)
     save_file(W, os.path.join(out_dir, "model.safetensors"))
     return out_dir
+
+
+def write_gosuvik(out_dir: str, width: int = 256, kinds=("channel_delta", "latent_attention", "parallel"), heads: int = 4,
+                  kv_heads: int = 2, dim: int = 64, vdim: int = 64, conv: int = 4, rank: int = 32, rot_dim: int = 32,
+                  kv_rank: int = 128, window: int = 256, r_heads: int = 2, r_dim: int = 64, r_vdim: int = 64, ff: int = 1024,
+                  experts: int = 0, top: int = 2, expert_ff: int = 256, groups: int = 4, loop=None, vocab: int = 32000,
+                  seed: int = 0) -> str:
+    """Random-init Gosuvik checkpoint directory (config.json + model.safetensors, bf16): one layer per
+    entry of `kinds` (the mixer types), all of the given sizes: the delta rule with `heads` heads over
+    `kv_heads` q / k heads and decay / gate projections of `rank`; latent attention with a latent of
+    kv_rank and a rotated part of rot_dim; the parallel mixer with grouped-query sink attention beside
+    a matrix memory of r_heads heads.  experts > 0: routed experts instead of the dense polynomial
+    feed-forward; loop = (start, stop, times).  Benchmarks and smoke runs; the weights mean nothing."""
+    import json
+
+    import torch
+    from safetensors.torch import save_file
+    os.makedirs(out_dir, exist_ok=True)
+    g = torch.Generator().manual_seed(seed)
+    D = width
+
+    def rnd(*shape, s):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * s).to(torch.bfloat16)
+
+    def lin(a, b):
+        return rnd(a, b, s=b ** -0.5)
+
+    def norm(k):
+        return (1.0 + rnd(k, s=0.05).float()).to(torch.bfloat16)
+
+    W = {"embed": rnd(vocab, D, s=0.5), "final.norm": norm(D), "head": lin(vocab, D)}
+    layers = []
+    for i, kind in enumerate(kinds):
+        p = f"l{i}.mix."
+        W[f"l{i}.norm1"], W[f"l{i}.norm2"] = norm(D), norm(D)
+        if kind == "channel_delta":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+            cq, cv = kv_heads * dim, heads * vdim
+            W[p + "q"], W[p + "k"], W[p + "v"], W[p + "b"] = lin(cq, D), lin(cq, D), lin(cv, D), lin(heads, D)
+            W[p + "q.conv"], W[p + "k.conv"], W[p + "v.conv"] = rnd(cq, conv, s=0.5), rnd(cq, conv, s=0.5), rnd(cv, conv, s=0.5)
+            W[p + "a1"], W[p + "a2"], W[p + "g1"], W[p + "g2"] = lin(rank, D), lin(heads * dim, rank), lin(rank, D), lin(cv, rank)
+            W[p + "dt_bias"] = (rnd(heads * dim, s=0.5).float() - 2.0).to(torch.bfloat16)
+            W[p + "A_log"], W[p + "norm"], W[p + "o"] = rnd(heads, s=0.5), norm(vdim), lin(D, cv)
+        elif kind == "latent_attention":
+            m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": (dim + rot_dim) ** -0.5,
+                 "mask": {"size": window},
+                 "rot": {"dims": rot_dim, "base": 10000.0, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+            W[p + "q"], W[p + "dkv"], W[p + "dkv.norm"] = lin(heads * (dim + rot_dim), D), lin(kv_rank + rot_dim, D), norm(kv_rank)
+            W[p + "uk"], W[p + "uv"] = lin(heads * dim, kv_rank), lin(heads * vdim, kv_rank)
+            W[p + "g"], W[p + "o"] = lin(heads * vdim, D), lin(D, heads * vdim)
+        elif kind == "parallel":
+            left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "mask": {"size": window},
+                    "rot": {"dims": dim // 2, "base": 10000.0, "scaling": {"factor": 2.0}}}
+            right = {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "gate_cap": 15.0}
+            m = {"left": left, "right": right, "left_scale": 0.5, "right_scale": 0.5}
+            q = p + "left."
+            W[q + "q"], W[q + "k"], W[q + "v"] = lin(heads * dim, D), lin(kv_heads * dim, D), lin(kv_heads * vdim, D)
+            W[q + "q.norm"], W[q + "k.norm"], W[q + "sink"], W[q + "o"] = norm(dim), norm(dim), rnd(heads, s=0.5), lin(D, heads * vdim)
+            q = p + "right."
+            W[q + "q"], W[q + "k"], W[q + "v"] = lin(r_heads * r_dim, D), lin(r_heads * r_dim, D), lin(r_heads * r_vdim, D)
+            W[q + "g"], W[q + "i"], W[q + "f"] = lin(r_heads * r_vdim, D), lin(r_heads, D), lin(r_heads, D)
+            W[q + "i.b"], W[q + "f.b"] = rnd(r_heads, s=0.5), (rnd(r_heads, s=0.5).float() + 3.0).to(torch.bfloat16)
+            W[q + "norm"], W[q + "o"] = norm(r_heads * r_vdim), lin(D, r_heads * r_vdim)
+        else:
+            raise ValueError(f"unknown mixer kind {kind!r}")
+        p = f"l{i}.mlp."
+        if experts:
+            f = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}
+            for e in range(experts):
+                W[p + f"e{e}.gate"], W[p + f"e{e}.up"], W[p + f"e{e}.down"] = lin(expert_ff, D), lin(expert_ff, D), lin(D, expert_ff)
+            W[p + "router"] = lin(experts, D)
+        else:
+            f = {"kind": "dense", "ff": ff}
+            W[p + "up"], W[p + "down"] = lin(ff, D), lin(D, ff)
+            W[p + "act"] = torch.tensor([0.6, 0.3, 0.1, 0.0]).to(torch.bfloat16)
+        layers.append({"type": kind, "mixer": m, "mlp": f})
+    cfg = {"architecture": "Gosuvik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": groups}, "layers": layers}
+    if loop:
+        cfg["loop"] = {"start": int(loop[0]), "stop": int(loop[1]), "times": int(loop[2])}
+    with open(os.path.join(out_dir, "config.json"), "w") as f_:
+        json.dump(cfg, f_)
+    save_file(W, os.path.join(out_dir, "model.safetensors"))
+    return out_dir

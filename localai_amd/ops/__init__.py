@@ -2734,7 +2734,7 @@ def qk_norm_rope_pages(src: torch.Tensor, H: int, D: int, G: int, Dv: int, pos: 
     q = torch.empty(T, Cq, dtype=src.dtype, device=src.device)
     _check(lib().la_qk_norm_rope_pages(int(src.dtype == torch.float32), src.data_ptr(), src.stride(0), T, H, D, G, Dv,
                                        pos.data_ptr(), slots.data_ptr(), q_w.data_ptr(), k_w.data_ptr(), float(eps),
-                                       freqs.data_ptr(), float(mag), rot, _ptr(v_freqs), q.data_ptr(), k_cache.data_ptr(),
+                                       _ptr(freqs) if rot else None, float(mag), rot, _ptr(v_freqs), q.data_ptr(), k_cache.data_ptr(),
                                        v_cache.data_ptr(), k_cache.shape[2], _stream()), "la_qk_norm_rope_pages")
     return q
 

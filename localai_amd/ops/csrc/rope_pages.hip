@@ -253,7 +253,7 @@ extern "C" int la_qk_norm_rope_pages(int f32, const void* src, long ld, int T, i
   using namespace la;
   if (T <= 0 || H <= 0 || D <= 0 || G <= 0 || Dv <= 0 || (rot & 1) || rot < 0 || rot > D || (vfreqs && (Dv & 1))) return -1;
   if (ld < (long)(H + G) * D + (long)G * Dv || BS <= 0 || (BS & 7)) return -2;
-  if (!src || !pos || !slots || !qw || !kw || !freqs || !q_out || !kc || !vc) return -3;
+  if (!src || !pos || !slots || !qw || !kw || (rot > 0 && !freqs) || !q_out || !kc || !vc) return -3;
   const size_t shm = (size_t)(rot + Dv + 2) * sizeof(float);
   if (f32)
     hipLaunchKernelGGL(qk_norm_rope_pages_kernel<float>, dim3(T), dim3(RP_NT), shm, (hipStream_t)stream, (const float*)src,

@@ -5,7 +5,8 @@ For each size two-layer models are built -- Suganex: dense feed-forwards (beside
 checkpoint) and routed experts (beside a Mixtral-style checkpoint); Dadizen: one model per mixer
 kind (windowed attention, latent attention, retention) beside the llama checkpoint; Vinozen:
 attention with a dense feed-forward, attention with routed experts, the state-space mixer, beside
-the llama and Mixtral-style checkpoints -- all stored as
+the llama and Mixtral-style checkpoints; Gosuvik: the delta rule, latent attention with routed experts,
+the parallel mixer, beside the same two -- all stored as
 dense bf16 weights so every GEMM takes the same library path, and each is timed through its engine's own
 batch construction (native scheduler, paged KV pool, state slots) and `model.forward`:
   prefill: `n_seq` prompts of `prompt` tokens in one batch, tokens/s;
@@ -87,6 +88,29 @@ def _vinozen_models(size: str, cache: str) -> Dict[str, str]:
                                 experts=s["experts"] if f == "moe" else 0, top=s["top"], expert_ff=s["eff"],
                                 side_dim=s["dim"], vocab=VOCAB)
         out[f"vinozen-{kind}"] = p
+    out["llama-dense"] = _llama(size, cache)
+    out["mixtral-moe"] = _llama(size, cache, moe=True)
+    return out
+
+
+def _gosuvik_models(size: str, cache: str) -> Dict[str, str]:
+    """Two equal layers each: the delta rule (as many q / k heads as heads, head width of the size, decay
+    and gate projections of one head width, 4 taps) with the dense polynomial feed-forward; latent
+    attention (latent 4 head widths, rotated part half a head width, window = the size's chunk) with
+    routed experts; the parallel mixer (grouped-query sink attention of the size's heads, window = the
+    size's chunk, beside a matrix memory of half as many heads) with the dense feed-forward."""
+    from ..models import synth
+    s = SIZES[size]
+    out = {}
+    for kind, moe in (("channel_delta", False), ("latent_attention", True), ("parallel", False)):
+        p = os.path.join(cache, f"gosuvik-{size}-{kind}")
+        if not os.path.exists(os.path.join(p, "model.safetensors")):
+            kv = s["heads"] if kind == "channel_delta" else s["kv"]
+            synth.write_gosuvik(p, width=s["width"], kinds=(kind, kind), heads=s["heads"], kv_heads=kv, dim=s["dim"],
+                                vdim=s["dim"], conv=4, rank=s["dim"], rot_dim=s["dim"] // 2, kv_rank=4 * s["dim"],
+                                window=s["chunk"], r_heads=max(1, s["heads"] // 2), r_dim=s["dim"], r_vdim=s["dim"], ff=s["ff"],
+                                experts=s["experts"] if moe else 0, top=s["top"], expert_ff=s["eff"], groups=4, vocab=VOCAB)
+        out[f"gosuvik-{kind}" + ("-moe" if moe else "-dense")] = p
     out["llama-dense"] = _llama(size, cache)
     out["mixtral-moe"] = _llama(size, cache, moe=True)
     return out
@@ -198,15 +222,16 @@ def _measure(path: str, n_seq: int, prompt: int, batch: int, context: int, iters
 
 def run(design: str, sizes: List[str], cache: str, n_seq: int = 4, prompt: int = 2048, batch: int = 64,
         context: int = 1536, iters: int = 5) -> dict:
-    if design not in ("suganex", "dadizen", "vinozen"):
-        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex, dadizen, vinozen)")
+    if design not in ("suganex", "dadizen", "vinozen", "gosuvik"):
+        raise SystemExit(f"--design-compare: unknown design {design!r} (suganex, dadizen, vinozen, gosuvik)")
     os.makedirs(cache, exist_ok=True)
     res = {"design": design, "dtype": "bf16", "data": "synthetic", "layers": 2,
            "workload": {"prefill": f"{n_seq} x {prompt} tokens", "decode": f"batch {batch} at context {context}"},
            "sizes": {}}
     for size in sizes:
         t0 = time.time()
-        paths = {"suganex": _models, "dadizen": _dadizen_models, "vinozen": _vinozen_models}[design](size, cache)
+        paths = {"suganex": _models, "dadizen": _dadizen_models, "vinozen": _vinozen_models,
+                 "gosuvik": _gosuvik_models}[design](size, cache)
         row = {}
         for name, p in paths.items():
             row[name] = {k: round(v, 3 if k.endswith("ms") else 1)
