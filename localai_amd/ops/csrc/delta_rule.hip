@@ -141,14 +141,14 @@ __global__ __launch_bounds__(DR_NT) void delta_tail_kernel(const AT* __restrict_
     if (i < taps - 1) st[(long)i * C + c] = nv[i];
 }
 
-template <int R, int C>
+template <int R, int C, int P>
 __global__ __launch_bounds__(DR_NT) void delta_scan_kernel(
     const float* __restrict__ qk, const float* __restrict__ vf, const float* __restrict__ gd, const float* __restrict__ bq,
     int H, int G, int Dk, int Dv, const int* __restrict__ pos, const int* __restrict__ cu_q,
-    const int* __restrict__ sslots, float* __restrict__ state, float* __restrict__ o, int P) {
+    const int* __restrict__ sslots, float* __restrict__ state, float* __restrict__ o) {
   extern __shared__ float lds[];
-  const int DkP = P * R;                 // padded key width (rows beyond Dk hold zeros)
-  const int cpw = DR_NT / P * C;         // value columns of this workgroup
+  constexpr int DkP = P * R;             // padded key width (rows beyond Dk hold zeros)
+  constexpr int cpw = DR_NT / P * C;     // value columns of this workgroup
   float* qs = lds;                       // [TC][DkP]
   float* ks = qs + DR_TC * DkP;          // [TC][DkP]
   float* gs = ks + DR_TC * DkP;          // [TC][DkP]
@@ -216,17 +216,22 @@ __global__ __launch_bounds__(DR_NT) void delta_scan_kernel(
           aq[ci] = fmaf(s, qj, aq[ci]);
         }
       }
+      // all 2 C sums move through every level of the butterfly together (the lane count is a template
+      // parameter: the exchanges unroll and overlap instead of forming one chain of dependent shuffles)
+#pragma unroll
+      for (int w = P >> 1; w > 0; w >>= 1) {
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) {
+          ak[ci] += __shfl_xor(ak[ci], w, 64);
+          aq[ci] += __shfl_xor(aq[ci], w, 64);
+        }
+      }
 #pragma unroll
       for (int ci = 0; ci < C; ++ci) {
-        float x = ak[ci], y = aq[ci];
-        for (int w = P >> 1; w > 0; w >>= 1) {
-          x += __shfl_xor(x, w, 64);
-          y += __shfl_xor(y, w, 64);
-        }
-        const float u = beta * (vs[tt * cpw + cg * C + ci] - x);
+        const float u = beta * (vs[tt * cpw + cg * C + ci] - ak[ci]);
 #pragma unroll
         for (int j = 0; j < R; ++j) S[ci][j] = fmaf(kj[j], u, S[ci][j]);
-        if (part == 0 && cb + ci < Dv) o[((long)(t0 + tt) * H + h) * Dv + cb + ci] = fmaf(u, kq, y);
+        if (part == 0 && cb + ci < Dv) o[((long)(t0 + tt) * H + h) * Dv + cb + ci] = fmaf(u, kq, aq[ci]);
       }
     }
   }
@@ -286,27 +291,35 @@ static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, i
   const int need = (Dk + P - 1) / P;
   const int cpw = DR_NT / P * Cc;
   const int nz = (Dv + cpw - 1) / cpw;
-#define LA_DR_LAUNCH(RR, CC)                                                                                         \
+#define LA_DR_LAUNCH(RR, CC, PP)                                                                                     \
   {                                                                                                                  \
-    const size_t shm = (size_t)(3 * DR_TC * P * RR + DR_TC * cpw + 2 * DR_TC) * sizeof(float);                       \
+    const size_t shm = (size_t)(3 * DR_TC * PP * RR + DR_TC * cpw + 2 * DR_TC) * sizeof(float);                      \
     if (shm > 150 * 1024) return -6;                                                                                 \
     if (shm > 48 * 1024)                                                                                             \
-      (void)hipFuncSetAttribute((const void*)delta_scan_kernel<RR, CC>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                                (int)shm);                                                                           \
-    hipLaunchKernelGGL((delta_scan_kernel<RR, CC>), dim3(nseq, H, nz), dim3(DR_NT), shm, st, (const float*)qk,       \
+      (void)hipFuncSetAttribute((const void*)delta_scan_kernel<RR, CC, PP>,                                          \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                               \
+    hipLaunchKernelGGL((delta_scan_kernel<RR, CC, PP>), dim3(nseq, H, nz), dim3(DR_NT), shm, st, (const float*)qk,   \
                        (const float*)vf, (const float*)gd, (const float*)bq, H, G, Dk, Dv, pos, cu_q, sslots, state, \
-                       o, P);                                                                                        \
+                       o);                                                                                           \
+  }
+#define LA_DR_P(RR, CC)                                                                                              \
+  {                                                                                                                  \
+    if (P == 8) LA_DR_LAUNCH(RR, CC, 8)                                                                              \
+    else if (P == 16) LA_DR_LAUNCH(RR, CC, 16)                                                                       \
+    else if (P == 32) LA_DR_LAUNCH(RR, CC, 32)                                                                       \
+    else LA_DR_LAUNCH(RR, CC, 64)                                                                                    \
   }
 #define LA_DR_R(CC)                                                                                                  \
   {                                                                                                                  \
-    if (need <= 1) LA_DR_LAUNCH(1, CC)                                                                               \
-    else if (need <= 2) LA_DR_LAUNCH(2, CC)                                                                          \
-    else if (need <= 4) LA_DR_LAUNCH(4, CC)                                                                          \
-    else if (need <= 8) LA_DR_LAUNCH(8, CC)                                                                          \
-    else LA_DR_LAUNCH(16, CC)                                                                                        \
+    if (need <= 1) LA_DR_P(1, CC)                                                                                    \
+    else if (need <= 2) LA_DR_P(2, CC)                                                                               \
+    else if (need <= 4) LA_DR_P(4, CC)                                                                               \
+    else if (need <= 8) LA_DR_P(8, CC)                                                                               \
+    else LA_DR_P(16, CC)                                                                                             \
   }
   if (Cc == 4) LA_DR_R(4)
   else LA_DR_R(1)
+#undef LA_DR_P
 #undef LA_DR_R
 #undef LA_DR_LAUNCH
   const long rows = (long)T * H;

@@ -12,9 +12,9 @@
 // State per sequence: [slots][H][Dv + 1][Dk] fp32 (value-column major, n last) and m [slots][H]; all zero
 // at position 0.
 //
-// mm_prep_kernel: fp32 rows [q Dk^-1/2 | k] and [v | 1] per head.   mm_gates_kernel: a thread per
-// (sequence portion, head) walks the portion's tokens for m (two operations a token on the chain; the
-// gate activations do not depend on it) and writes (a_t, s_t, exp(-m_t)).   mm_out_kernel: denominator,
+// mm_prep_kernel: fp32 rows [q Dk^-1/2 | k] and [v | 1] per head.   mm_gates_kernel: a wave per
+// (sequence portion, head) finds m for 64 tokens at a time by a scan over the lanes and writes
+// (a_t, s_t, exp(-m_t)).   mm_out_kernel: denominator,
 // unit norm, weight, gate, scale; a wave per (token, head).
 #include "common.h"
 
@@ -43,32 +43,51 @@ __global__ __launch_bounds__(256) void mm_prep_kernel(const AT* __restrict__ src
 
 LA_DEV float log_sigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
+// A wave per (sequence portion, head), 64 tokens at a time: a token is the map m -> max(m + f, i), maps
+// compose as (F1, I1) then (F2, I2) = (F1 + F2, max(I1 + F2, I2)), so an inclusive scan over the lanes
+// gives every token's m from the chunk's incoming m.
 template <typename AT>
 __global__ __launch_bounds__(64) void mm_gates_kernel(const AT* __restrict__ src, long ld, int gcol, int H, int nseq,
                                                       const float* __restrict__ gate_b, float cap,
                                                       const int* __restrict__ pos, const int* __restrict__ cu_q,
                                                       const int* __restrict__ sslots, float* __restrict__ mstate,
                                                       float* __restrict__ gts) {
-  const int e = blockIdx.x * 64 + threadIdx.x;
-  if (e >= nseq * H) return;
-  const int seq = e / H, h = e - seq * H;
+  const int seq = blockIdx.x / H, h = blockIdx.x - seq * H, lane = threadIdx.x;
   const int a = cu_q[seq], b = cu_q[seq + 1];
   if (b <= a) return;
   const int slot = sslots[seq];
-  float m = (slot >= 0 && pos[a] != 0) ? mstate[(long)slot * H + h] : 0.f;
+  float m0 = (slot >= 0 && pos[a] != 0) ? mstate[(long)slot * H + h] : 0.f;
   const float bi = gate_b[h], bf = gate_b[H + h];
-  for (int t = a; t < b; ++t) {
-    const AT* row = src + (long)t * ld + gcol;
-    const float ig = cap * tanhf(((float)row[h] + bi) / cap);
-    const float fg = log_sigmoid(cap * tanhf(((float)row[H + h] + bf) / cap));
-    const float m2 = fmaxf(fg + m, ig);
-    float* g = gts + (long)t * 3 * H;
-    g[h] = expf(fg + m - m2);
-    g[H + h] = expf(ig - m2);
-    g[2 * H + h] = expf(-m2);
-    m = m2;
+  for (int t0 = a; t0 < b; t0 += 64) {
+    const int t = t0 + lane;
+    const bool live = t < b;
+    float ig = -INFINITY, fg = 0.f;        // a lane past the end is the identity map
+    if (live) {
+      const AT* row = src + (long)t * ld + gcol;
+      ig = cap * tanhf(((float)row[h] + bi) / cap);
+      fg = log_sigmoid(cap * tanhf(((float)row[H + h] + bf) / cap));
+    }
+    float F = fg, I = ig;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float Fp = __shfl_up(F, off, 64), Ip = __shfl_up(I, off, 64);
+      if (lane >= off) {
+        I = fmaxf(Ip + F, I);
+        F = Fp + F;
+      }
+    }
+    const float m = fmaxf(m0 + F, I);
+    float mp = __shfl_up(m, 1, 64);
+    if (lane == 0) mp = m0;
+    if (live) {
+      float* g = gts + (long)t * 3 * H;
+      g[h] = expf(fg + mp - m);
+      g[H + h] = expf(ig - m);
+      g[2 * H + h] = expf(-m);
+    }
+    m0 = __shfl(m, min(63, b - 1 - t0), 64);
   }
-  if (slot >= 0) mstate[(long)slot * H + h] = m;
+  if (slot >= 0 && lane == 0) mstate[(long)slot * H + h] = m0;
 }
 
 template <typename AT>
@@ -106,7 +125,7 @@ static int mm_launch(const AT* src, long ld, int T, int nseq, int H, int Dk, int
   hipLaunchKernelGGL(mm_prep_kernel<AT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src, ld, H, Dk, Dv,
                      1.f / sqrtf((float)Dk), qk, va, total);
   const int gcol = 2 * H * Dk + 2 * H * Dv;
-  hipLaunchKernelGGL(mm_gates_kernel<AT>, dim3((nseq * H + 63) / 64), dim3(64), 0, st, src, ld, gcol, H, nseq, gate_b, cap,
+  hipLaunchKernelGGL(mm_gates_kernel<AT>, dim3(nseq * H), dim3(64), 0, st, src, ld, gcol, H, nseq, gate_b, cap,
                      pos, cu_q, sslots, mstate, gts);
   const int rc = decay_scan_f32(va, H * (Dv + 1), qk, T, nseq, H, H, Dk, Dv + 1, pos, cu_q, sslots, mem, gts, gts + H, 3 * H,
                                 o, seg, max_rows, st);
