@@ -41,6 +41,31 @@ LA_DEV int portion_of(const int* __restrict__ cu_q, int nseq, int t) {
   return lo;
 }
 
+
+// The value of lane (l xor W).  Within a row of 16 lanes the exchange is a data-parallel move on the
+// vector unit (quad permutes and mirrors composed: i -> 7 - i -> i xor 4, i -> 15 - i -> i xor 8), which
+// keeps the scan's reductions off the LDS crossbar; wider exchanges go through it.
+template <int CTRL>
+LA_DEV float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int W>
+LA_DEV float lane_xor(float v) {
+  if constexpr (W == 1) return dpp_move<0xB1>(v);                        // quad_perm [1, 0, 3, 2]
+  else if constexpr (W == 2) return dpp_move<0x4E>(v);                   // quad_perm [2, 3, 0, 1]
+  else if constexpr (W == 4) return dpp_move<0x1B>(dpp_move<0x141>(v));  // row_half_mirror, then quad_perm [3, 2, 1, 0]
+  else if constexpr (W == 8) return dpp_move<0x141>(dpp_move<0x140>(v)); // row_mirror, then row_half_mirror
+  else return __shfl_xor(v, W, 64);
+}
+template <int W, int N>
+LA_DEV void butterfly_level(float (&a)[N], float (&b)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    a[i] += lane_xor<W>(a[i]);
+    b[i] += lane_xor<W>(b[i]);
+  }
+}
+
 template <typename AT>
 __global__ __launch_bounds__(DR_NT) void delta_prep_kernel(
     const AT* __restrict__ src, long ld, const AT* __restrict__ dec, int H, int G, int Dk, int Dv, int taps,
@@ -218,14 +243,12 @@ __global__ __launch_bounds__(DR_NT) void delta_scan_kernel(
       }
       // all 2 C sums move through every level of the butterfly together (the lane count is a template
       // parameter: the exchanges unroll and overlap instead of forming one chain of dependent shuffles)
-#pragma unroll
-      for (int w = P >> 1; w > 0; w >>= 1) {
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci) {
-          ak[ci] += __shfl_xor(ak[ci], w, 64);
-          aq[ci] += __shfl_xor(aq[ci], w, 64);
-        }
-      }
+      if constexpr (P >= 64) butterfly_level<32, C>(ak, aq);
+      if constexpr (P >= 32) butterfly_level<16, C>(ak, aq);
+      if constexpr (P >= 16) butterfly_level<8, C>(ak, aq);
+      butterfly_level<4, C>(ak, aq);
+      butterfly_level<2, C>(ak, aq);
+      butterfly_level<1, C>(ak, aq);
 #pragma unroll
       for (int ci = 0; ci < C; ++ci) {
         const float u = beta * (vs[tt * cpw + cg * C + ci] - ak[ci]);
@@ -282,12 +305,14 @@ static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, i
                        cu_q, sslots, tail);
   // P lanes per group of Cc value columns (power of two), R rows per lane: P * R >= Dk; a thread keeps
   // Cc x R state entries.  More lanes per group while the launch has fewer than about four workgroups
-  // per compute unit: a scan is a chain of dependent steps, so resident waves hide its latencies.
+  // per compute unit (a scan is a chain of dependent steps, so resident waves hide its latencies), up to
+  // 32: the sixth butterfly level costs more than the wider launch gains (4 x 2048 rows, 16 heads of
+  // 128 x 128: 2.5 ms with 32 lanes, 3.3 ms with 64).
   const int Cc = Dv >= 64 ? 4 : 1;
   int P = 8;
   while (P < 64 && (Dk + P - 1) / P > (Cc == 4 ? 8 : 16)) P <<= 1;
   if ((Dk + P - 1) / P > 16) return -5;
-  while (P < 64 && (Dk + P - 1) / P > 2 && (long)nseq * H * ((Dv + DR_NT / P * Cc - 1) / (DR_NT / P * Cc)) < 1024) P <<= 1;
+  while (P < 32 && (Dk + P - 1) / P > 2 && (long)nseq * H * ((Dv + DR_NT / P * Cc - 1) / (DR_NT / P * Cc)) < 1024) P <<= 1;
   const int need = (Dk + P - 1) / P;
   const int cpw = DR_NT / P * Cc;
   const int nz = (Dv + cpw - 1) / cpw;
