@@ -187,6 +187,7 @@ class _Layer:
     rank_a: int = 0
     rank_g: int = 0
     conv: Optional[torch.Tensor] = None          # fp32 [C, taps]
+    conv_t: Optional[torch.Tensor] = None        # the same tap-major, [taps, C] (the vectorised kernel's layout)
     dt_bias: Optional[torch.Tensor] = None
     a_log: Optional[torch.Tensor] = None
     mix_norm: Optional[torch.Tensor] = None
@@ -300,6 +301,7 @@ class GosuvikModel:
         L.rank_a, L.rank_g = ra, rg
         L.conv = torch.cat([sh(p + "q.conv", (Cqk, m.taps)), sh(p + "k.conv", (Cqk, m.taps)),
                             sh(p + "v.conv", (Cv, m.taps))], 0).to(self.device).contiguous()
+        L.conv_t = L.conv.t().contiguous()
         L.dt_bias = self._f32(p + "dt_bias", (H * m.dim,))
         L.a_log = self._f32(p + "A_log", (H,))
         L.mix_norm = self._f32(p + "norm", (m.vdim,))
@@ -453,7 +455,7 @@ class GosuvikModel:
         conv_state, rec_state = kv.state[run]
         return ops.delta_rule(proj, dec, gate, m.heads, m.kv_heads, m.dim, m.vdim, L.conv, L.dt_bias, L.a_log, L.mix_norm,
                               self.hp.norm_eps, fb.pos, cu_q, fb.sslots, conv_state, rec_state, UNIT_EPS,
-                              max_rows=1 if fb.decode else fb.max_q)
+                              max_rows=1 if fb.decode else fb.max_q, conv_wt=L.conv_t)
 
     def _latent(self, L: _Layer, m: MixSpec, xn, fb, kv, run, row_seq, splits: int = 1):
         T, H, r, dn, dr = xn.shape[0], m.heads, m.kv_rank, m.dim, m.rot_dim

@@ -138,8 +138,8 @@ def lib():
             "la_sigmoid_mul": [P, I, P, I, LNG, I, I, P, I, P],
             "la_qk_norm_rope_pages": [I, P, LNG, I, I, I, I, I, P, P, P, P, F, P, F, I, P, P, P, P, I, P],
             "la_rotate_heads": [I, P, I, I, I, P, P, F, F, P, LNG, P],
-            "la_delta_rule": [I, P, LNG, P, P, I, I, I, I, I, I, I, I, P, P, P, P, F, F, P, P, P, P, P, I, P, P, P, P, P,
-                              P, P],
+            "la_delta_rule": [I, P, LNG, P, P, I, I, I, I, I, I, I, I, P, P, P, P, P, F, F, P, P, P, P, P, I, P, P, P, P,
+                              P, P, P],
             "la_matrix_memory": [I, P, LNG, I, I, I, I, I, P, F, P, F, F, F, P, P, P, P, P, I, P, P, P, P, P, LNG, P, I,
                                  P],
             "la_glu_clamp": [P, I, LNG, I, I, I, F, F, P, I, P],
@@ -2788,7 +2788,8 @@ def delta_rule_states(slots: int, H: int, G: int, Dk: int, Dv: int, taps: int, d
 def delta_rule(src: torch.Tensor, dec: torch.Tensor, gate: torch.Tensor, H: int, G: int, Dk: int, Dv: int,
                conv_w: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, norm_w: torch.Tensor, eps: float,
                pos: torch.Tensor, cu_q: torch.Tensor, sslots: torch.Tensor, conv_state: torch.Tensor,
-               rec_state: torch.Tensor, unit_eps: float = 1e-6, max_rows: int = 0) -> torch.Tensor:
+               rec_state: torch.Tensor, unit_eps: float = 1e-6, max_rows: int = 0,
+               conv_wt: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Gated delta rule with one decay per head and key channel over projection rows src [T, >= 2 G
     Dk + H Dv + H] laid out [q | k | v | beta logits] (any row stride), dec [T, H Dk] (decay
     logits) and gate [T, H Dv] (output gate logits):
@@ -2804,7 +2805,9 @@ def delta_rule(src: torch.Tensor, dec: torch.Tensor, gate: torch.Tensor, H: int,
     comes from conv_state[sslots[seq]] (the last taps - 1 rows of [q | k | v] before the
     convolution) and rec_state[sslots[seq]] (fp32 [H, Dv, Dk]), both taken as zero before position
     0, and both are advanced to the portion's end.  Everything after the convolution's silu is
-    fp32.  Returns [T, H Dv] in src's dtype."""
+    fp32.  conv_wt: conv_w tap-major ([taps, C] fp32), which the vectorised bf16 kernel reads (key and
+    value widths and the row stride multiples of 8); made per call when not given.  Returns [T, H Dv]
+    in src's dtype."""
     T = src.shape[0]
     nseq = cu_q.shape[0] - 1
     Cqk, Cv = G * Dk, H * Dv
@@ -2861,6 +2864,10 @@ def delta_rule(src: torch.Tensor, dec: torch.Tensor, gate: torch.Tensor, H: int,
     for t in (conv_w, dt_bias, a_log, norm_w):
         assert t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda
     dev = src.device
+    if conv_wt is None and not f32 and not (Dk % 8 or Dv % 8 or src.stride(0) % 8):
+        conv_wt = conv_w.t().contiguous()
+    if conv_wt is not None and (conv_wt.dtype != torch.float32 or tuple(conv_wt.shape) != (taps, C) or not conv_wt.is_contiguous()):
+        raise ValueError("delta_rule: conv_wt must be the fp32 [taps, C] transpose of conv_w")
     qk = torch.empty(T, 2 * Cqk, dtype=torch.float32, device=dev)       # unit q (scaled) | unit k per group
     vf = torch.empty(T, Cv, dtype=torch.float32, device=dev)            # convolved v
     gd = torch.empty(T, H * Dk, dtype=torch.float32, device=dev)        # decays per (token, head, key channel)
@@ -2869,7 +2876,7 @@ def delta_rule(src: torch.Tensor, dec: torch.Tensor, gate: torch.Tensor, H: int,
     out = torch.empty(T, Cv, dtype=src.dtype, device=dev)
     max_rows = int(max_rows) if max_rows > 0 else T
     _check(lib().la_delta_rule(int(f32), src.data_ptr(), src.stride(0), dec.data_ptr(), gate.data_ptr(), T, nseq, H, G, Dk,
-                               Dv, taps, rec_state.shape[0], conv_w.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(),
+                               Dv, taps, rec_state.shape[0], conv_w.data_ptr(), _ptr(conv_wt), dt_bias.data_ptr(), a_log.data_ptr(),
                                norm_w.data_ptr(), float(eps), float(unit_eps), pos.data_ptr(), cu_q.data_ptr(),
                                sslots.data_ptr(), conv_state.data_ptr(), rec_state.data_ptr(),
                                int(T == nseq and max_rows == 1), qk.data_ptr(), vf.data_ptr(), gd.data_ptr(), bq.data_ptr(),

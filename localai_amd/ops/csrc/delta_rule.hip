@@ -14,7 +14,8 @@
 //   the portion's rows, then from the tail, zeros before position 0); a wave per q / k group forms both
 //   unit vectors and k . q; fp32 rows out: [q | k] per group, v, the decays, (beta | k . q).  Batches of one
 //   row per sequence advance the tail in the same launch (a thread owns its channels), other batches in
-//   delta_tail_kernel afterwards, since rows of a portion read the old tail.
+//   delta_tail_kernel afterwards, since rows of a portion read the old tail.  delta_prep8_kernel: the same
+//   for bf16 rows of widths % 8, 8 channels a thread with 16-byte accesses and tap-major weights.
 // delta_scan_kernel: workgroup = (sequence portion, head, slice of value columns).  The columns of S are
 //   independent chains: column c needs a_c = (g S_c) . k and b_c = (g S_c) . q, then u_c = beta (v_c - a_c),
 //   S_c <- g S_c + k u_c, and o_c = b_c + u_c (k . q), which is S_c . q after the write.  A column's Dk
@@ -135,6 +136,106 @@ __global__ __launch_bounds__(DR_NT) void delta_prep_kernel(
     const int h = e / Dk;
     const float dt = dr_softplus((float)dec[(long)t * H * Dk + e] + dt_bias[e]);
     gd[(long)t * H * Dk + e] = expf(-expf(a_log[h]) * dt);
+  }
+}
+
+// The same step for bf16 rows whose widths are multiples of 8 (key and value widths, the row stride): a
+// thread takes 8 consecutive channels with 16-byte loads and reads the weights tap-major, w_t [taps][C],
+// so a row's loads are in flight together instead of one round trip per channel.
+__global__ __launch_bounds__(DR_NT) void delta_prep8_kernel(
+    const bf16* __restrict__ src, long ld, const bf16* __restrict__ dec, int H, int G, int Dk, int Dv, int taps,
+    const float* __restrict__ w_t, const float* __restrict__ dt_bias, const float* __restrict__ a_log, float unit_eps,
+    const int* __restrict__ pos, const int* __restrict__ cu_q, int nseq, const int* __restrict__ sslots,
+    bf16* __restrict__ tail, int single, float* __restrict__ qk, float* __restrict__ vf, float* __restrict__ gd,
+    float* __restrict__ bq) {
+  extern __shared__ float cv[];        // [C] convolved, activated channels of this token
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int Cqk = G * Dk, Cv = H * Dv, C = 2 * Cqk + Cv;
+  const int seq = single ? t : portion_of(cu_q, nseq, t);
+  const int a = cu_q[seq], p = pos[t], p0 = pos[a];
+  const int slot = sslots[seq];
+  const bf16* st = (slot >= 0 && taps > 1) ? tail + (long)slot * (taps - 1) * C : nullptr;
+  for (int c = tid * 8; c < C; c += DR_NT * 8) {
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    bf16x8 cur[DR_MAXTAPS];
+#pragma unroll
+    for (int j = 0; j < DR_MAXTAPS; ++j) {
+      if (j < taps) {
+        const int pj = p - (taps - 1) + j;
+        bf16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+        if (pj >= p0) v = *(const bf16x8*)(src + (long)(a + pj - p0) * ld + c);
+        else if (pj >= 0 && st) v = *(const bf16x8*)(st + (long)(pj - p0 + taps - 1) * C + c);
+        cur[j] = v;
+        const float4 w0 = *(const float4*)(w_t + (long)j * C + c), w1 = *(const float4*)(w_t + (long)j * C + c + 4);
+        acc[0] = fmaf(w0.x, (float)v[0], acc[0]);
+        acc[1] = fmaf(w0.y, (float)v[1], acc[1]);
+        acc[2] = fmaf(w0.z, (float)v[2], acc[2]);
+        acc[3] = fmaf(w0.w, (float)v[3], acc[3]);
+        acc[4] = fmaf(w1.x, (float)v[4], acc[4]);
+        acc[5] = fmaf(w1.y, (float)v[5], acc[5]);
+        acc[6] = fmaf(w1.z, (float)v[6], acc[6]);
+        acc[7] = fmaf(w1.w, (float)v[7], acc[7]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[i] = acc[i] / (1.f + expf(-acc[i]));
+      cv[c + i] = acc[i];
+    }
+    if (c >= 2 * Cqk) {
+      float4* o4 = (float4*)(vf + (long)t * Cv + (c - 2 * Cqk));
+      o4[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      o4[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
+    if (single && slot >= 0 && taps > 1) {      // one row per sequence: the tail moves on by one position
+      bf16* sw = tail + (long)slot * (taps - 1) * C;
+#pragma unroll
+      for (int j = 1; j < DR_MAXTAPS; ++j)
+        if (j < taps) *(bf16x8*)(sw + (long)(j - 1) * C + c) = cur[j];
+    }
+  }
+  __syncthreads();
+  const float qscale = 1.f / sqrtf((float)Dk);
+  for (int g = wave; g < G; g += DR_NT / 64) {
+    const float* q = cv + (long)g * Dk;
+    const float* k = cv + Cqk + (long)g * Dk;
+    float sq = 0.f, sk = 0.f, dot = 0.f;
+    for (int d = lane; d < Dk; d += 64) {
+      sq = fmaf(q[d], q[d], sq);
+      sk = fmaf(k[d], k[d], sk);
+      dot = fmaf(q[d], k[d], dot);
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    dot = wave_sum(dot);
+    const float iq = qscale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
+    float* qo = qk + ((long)t * 2 * G + g) * Dk;
+    float* ko = qo + (long)G * Dk;
+    for (int d = lane; d < Dk; d += 64) {
+      qo[d] = q[d] * iq;
+      ko[d] = k[d] * ik;
+    }
+    if (lane == 0) bq[(long)t * (H + G) + H + g] = dot * iq * ik;
+  }
+  for (int h = tid; h < H; h += DR_NT) {
+    const float b = (float)src[(long)t * ld + C + h];
+    bq[(long)t * (H + G) + h] = 1.f / (1.f + expf(-b));
+  }
+  for (int e = tid * 8; e < H * Dk; e += DR_NT * 8) {
+    const float ea = expf(a_log[e / Dk]);          // Dk % 8 == 0: the 8 channels share a head
+    const bf16x8 dv = *(const bf16x8*)(dec + (long)t * H * Dk + e);
+    const float4 b0 = *(const float4*)(dt_bias + e), b1 = *(const float4*)(dt_bias + e + 4);
+    const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = expf(-ea * dr_softplus((float)dv[i] + bb[i]));
+    float4* o4 = (float4*)(gd + (long)t * H * Dk + e);
+    o4[0] = make_float4(r[0], r[1], r[2], r[3]);
+    o4[1] = make_float4(r[4], r[5], r[6], r[7]);
   }
 }
 
@@ -290,16 +391,28 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
 
 template <typename AT>
 static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, int T, int nseq, int H, int G, int Dk, int Dv,
-                        int taps, const float* w, const float* dt_bias, const float* a_log, const float* nw, float eps,
+                        int taps, const float* w, const float* w_t, const float* dt_bias, const float* a_log, const float* nw, float eps,
                         float unit_eps, const int* pos, const int* cu_q, const int* sslots, AT* tail, float* state,
                         int single, float* qk, float* vf, float* gd, float* bq, float* o, AT* out, hipStream_t st) {
   const int C = 2 * G * Dk + H * Dv;
   const size_t shm0 = (size_t)C * sizeof(float);
   if (shm0 > 150 * 1024) return -6;
-  if (shm0 > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)delta_prep_kernel<AT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm0);
-  hipLaunchKernelGGL(delta_prep_kernel<AT>, dim3(T), dim3(DR_NT), shm0, st, src, ld, dec, H, G, Dk, Dv, taps, w, dt_bias,
-                     a_log, unit_eps, pos, cu_q, nseq, sslots, tail, single, qk, vf, gd, bq);
+  bool wide = false;
+  if constexpr (sizeof(AT) == 2)
+    wide = w_t && (Dk & 7) == 0 && (Dv & 7) == 0 && (ld & 7) == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)dec & 15) == 0;
+  if (wide) {
+    if constexpr (sizeof(AT) == 2) {
+      if (shm0 > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)delta_prep8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm0);
+      hipLaunchKernelGGL(delta_prep8_kernel, dim3(T), dim3(DR_NT), shm0, st, (const bf16*)src, ld, (const bf16*)dec, H, G, Dk,
+                         Dv, taps, w_t, dt_bias, a_log, unit_eps, pos, cu_q, nseq, sslots, (bf16*)tail, single, qk, vf, gd, bq);
+    }
+  } else {
+    if (shm0 > 48 * 1024)
+      (void)hipFuncSetAttribute((const void*)delta_prep_kernel<AT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm0);
+    hipLaunchKernelGGL(delta_prep_kernel<AT>, dim3(T), dim3(DR_NT), shm0, st, src, ld, dec, H, G, Dk, Dv, taps, w, dt_bias,
+                       a_log, unit_eps, pos, cu_q, nseq, sslots, tail, single, qk, vf, gd, bq);
+  }
   if (!single && taps > 1)
     hipLaunchKernelGGL(delta_tail_kernel<AT>, dim3(nseq, (C + DR_NT - 1) / DR_NT), dim3(DR_NT), 0, st, src, ld, C, taps, pos,
                        cu_q, sslots, tail);
@@ -356,7 +469,8 @@ static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, i
 }  // namespace la
 
 extern "C" int la_delta_rule(int f32, const void* src, long ld, const void* dec, const void* gate, int T, int nseq, int H,
-                             int G, int Dk, int Dv, int taps, int nslots, const void* conv_w, const void* dt_bias,
+                             int G, int Dk, int Dv, int taps, int nslots, const void* conv_w, const void* conv_wt,
+                             const void* dt_bias,
                              const void* a_log, const void* norm_w, float eps, float unit_eps, const void* pos,
                              const void* cu_q, const void* sslots, void* tail, void* state, int single, void* qk, void* vf,
                              void* gd, void* bq, void* o, void* out, void* stream) {
@@ -371,12 +485,12 @@ extern "C" int la_delta_rule(int f32, const void* src, long ld, const void* dec,
   hipStream_t st = (hipStream_t)stream;
   if (f32)
     return delta_launch<float>((const float*)src, ld, (const float*)dec, (const float*)gate, T, nseq, H, G, Dk, Dv, taps,
-                               (const float*)conv_w, (const float*)dt_bias, (const float*)a_log, (const float*)norm_w, eps,
-                               unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (float*)tail,
+                               (const float*)conv_w, (const float*)conv_wt, (const float*)dt_bias, (const float*)a_log,
+                               (const float*)norm_w, eps, unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (float*)tail,
                                (float*)state, single, (float*)qk, (float*)vf, (float*)gd, (float*)bq, (float*)o,
                                (float*)out, st);
   return delta_launch<bf16>((const bf16*)src, ld, (const bf16*)dec, (const bf16*)gate, T, nseq, H, G, Dk, Dv, taps,
-                            (const float*)conv_w, (const float*)dt_bias, (const float*)a_log, (const float*)norm_w, eps,
-                            unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (bf16*)tail, (float*)state,
+                            (const float*)conv_w, (const float*)conv_wt, (const float*)dt_bias, (const float*)a_log,
+                            (const float*)norm_w, eps, unit_eps, (const int*)pos, (const int*)cu_q, (const int*)sslots, (bf16*)tail, (float*)state,
                             single, (float*)qk, (float*)vf, (float*)gd, (float*)bq, (float*)o, (bf16*)out, st);
 }

@@ -8,6 +8,10 @@
 //     one launch where a pre-normed stream has "add + norm": the branch's own norm, the residual
 //     add and the next sublayer's input norm.  A workgroup per row; the rms variant reads the
 //     branch row twice (second time from cache) instead of holding it in registers, so any width runs.
+//   add_group_norm:  res += branch;  out = res normed in equal consecutive groups (each / its own rms) times w:
+//     the boundary of a pre-normed fp32 stream whose norm works on groups
+//   poly_norm_act:   y = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e over a row
+//   sigmoid_mul:     x * sigmoid(gate), the gate being columns of a wider row
 //   glu_clamp:   g = min(gate, limit), u = clamp(up, -limit, limit), y = g sigmoid(slope g) (u + 1)
 //   side_gate:   gelu_tanh(z[t][c]) * table[tok[t]][col0 + c]
 //
@@ -301,6 +305,52 @@ __global__ __launch_bounds__(NC_NT) void poly_norm_act_kernel(RowSrc src, int F,
   }
 }
 
+// The same for one bf16 matrix with F % 8 == 0 and F <= 16384: a thread keeps its columns (up to 8 vectors
+// of 8) in registers between the two passes, 16-byte loads and stores, the row is read once.
+constexpr int PN_MAXV = 8;
+__global__ __launch_bounds__(NC_NT) void poly_norm_act8_kernel(const bf16* __restrict__ src, int F,
+                                                               const float* __restrict__ coef, float eps,
+                                                               bf16* __restrict__ out) {
+  __shared__ float red[NC_NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x, nv = F >> 3;
+  const bf16x8* row = (const bf16x8*)(src + (long)t * F);
+  bf16x8 z[PN_MAXV];
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int k = 0; k < PN_MAXV; ++k) {
+    const int v = tid + k * NC_NT;
+    if (v < nv) {
+      z[k] = row[v];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = (float)z[k][j], x2 = x * x;
+        s2 += x2;
+        s4 = fmaf(x2, x2, s4);
+        s6 = fmaf(x2 * x2, x2, s6);
+      }
+    }
+  }
+  s2 = block_sum<NC_NT>(s2, red);
+  s4 = block_sum<NC_NT>(s4, red);
+  s6 = block_sum<NC_NT>(s6, red);
+  const float i1 = coef[0] / sqrtf(s2 / (float)F + eps), i2 = coef[1] / sqrtf(s4 / (float)F + eps),
+              i3 = coef[2] / sqrtf(s6 / (float)F + eps), e = coef[3];
+  bf16x8* orow = (bf16x8*)(out + (long)t * F);
+#pragma unroll
+  for (int k = 0; k < PN_MAXV; ++k) {
+    const int v = tid + k * NC_NT;
+    if (v < nv) {
+      bf16x8 y;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = (float)z[k][j];
+        y[j] = (bf16)fmaf(x, i1, fmaf(x * x, i2, fmaf(x * x * x, i3, e)));
+      }
+      orow[v] = y;
+    }
+  }
+}
+
 // out = x * sigmoid(gate), gate rows with their own stride (columns of a wider projection)
 __global__ __launch_bounds__(256) void sigmoid_mul_kernel(const void* __restrict__ x, int x_f32, const void* __restrict__ g,
                                                           int g_f32, long ldg, int N, long total, void* __restrict__ out,
@@ -312,6 +362,21 @@ __global__ __launch_bounds__(256) void sigmoid_mul_kernel(const void* __restrict
   const float xv = x_f32 ? ((const float*)x)[e] : (float)((const bf16*)x)[e];
   const float gv = g_f32 ? ((const float*)g)[t * ldg + c] : (float)((const bf16*)g)[t * ldg + c];
   put(out, out_f32, e, xv / (1.f + expf(-gv)));
+}
+
+// bf16 operands with N % 8 == 0 and 16-byte aligned rows: 8 columns a thread
+__global__ __launch_bounds__(256) void sigmoid_mul8_kernel(const bf16* __restrict__ x, const bf16* __restrict__ g, long ldg,
+                                                           int N, long total8, bf16* __restrict__ out) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total8) return;
+  const int nv = N >> 3;
+  const long t = e / nv;
+  const int c = (int)(e - t * nv) * 8;
+  const bf16x8 xv = *(const bf16x8*)(x + t * N + c), gv = *(const bf16x8*)(g + t * ldg + c);
+  bf16x8 y;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = (bf16)((float)xv[j] / (1.f + expf(-(float)gv[j])));
+  *(bf16x8*)(out + t * N + c) = y;
 }
 
 }  // namespace la
@@ -336,6 +401,11 @@ extern "C" int la_poly_norm_act(const void* sp, int src_f32, long slab, int S, i
                                 void* out, int out_f32, void* stream) {
   using namespace la;
   if (T <= 0 || F <= 0 || !sp || !coef || !out) return -1;
+  if (!src_f32 && !out_f32 && (F & 7) == 0 && F <= 8 * NC_NT * PN_MAXV) {
+    hipLaunchKernelGGL(poly_norm_act8_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, (const bf16*)sp, F,
+                       (const float*)coef, eps, (bf16*)out);
+    return (int)hipGetLastError();
+  }
   RowSrc s{sp, src_f32, slab, S};
   hipLaunchKernelGGL(poly_norm_act_kernel, dim3(T), dim3(NC_NT), 0, (hipStream_t)stream, s, F, (const float*)coef, eps, out,
                      out_f32);
@@ -346,6 +416,12 @@ extern "C" int la_sigmoid_mul(const void* x, int x_f32, const void* g, int g_f32
                               int out_f32, void* stream) {
   using namespace la;
   if (T <= 0 || N <= 0 || !x || !g || !out || ldg < N) return -1;
+  if (!x_f32 && !g_f32 && !out_f32 && (N & 7) == 0 && (ldg & 7) == 0 && (((uintptr_t)x | (uintptr_t)g | (uintptr_t)out) & 15) == 0) {
+    const long total8 = (long)T * (N >> 3);
+    hipLaunchKernelGGL(sigmoid_mul8_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16*)x, (const bf16*)g, ldg, N, total8, (bf16*)out);
+    return (int)hipGetLastError();
+  }
   const long total = (long)T * N;
   hipLaunchKernelGGL(sigmoid_mul_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, x_f32,
                      g, g_f32, ldg, N, total, out, out_f32);

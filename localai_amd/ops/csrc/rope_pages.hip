@@ -176,8 +176,17 @@ __global__ __launch_bounds__(RP_NT) void qk_norm_rope_pages_kernel(
   const int Cq = H * D, Ck = G * D, Cv = G * Dv, half = rot >> 1, vhalf = Dv >> 1;
   const AT* row = src + (long)t * ld;
   const int p = pos[t];
-  fill_cos_sin(cs, rot, p, freqs, mag);
-  if (vfreqs) fill_cos_sin(vcs, Dv, p, vfreqs, 1.f);
+  // both tables in one pass, a thread per angle, sine and cosine from one evaluation
+  for (int i = tid; i < half + (vfreqs ? vhalf : 0); i += RP_NT) {
+    const bool isv = i >= half;
+    const int k = isv ? i - half : i;
+    float sn, c;
+    sincosf((float)p * (isv ? vfreqs[k] : freqs[k]), &sn, &c);
+    float* dst = isv ? vcs : cs;
+    const float m = isv ? 1.f : mag;
+    dst[2 * k] = c * m;
+    dst[2 * k + 1] = sn * m;
+  }
   __syncthreads();
   const int slot = slots[t];
   const int blk = slot >= 0 ? slot / BS : 0, off = slot >= 0 ? slot - blk * BS : 0;
@@ -230,9 +239,10 @@ __global__ __launch_bounds__(RP_NT) void rotate_heads_kernel(const AT* __restric
   extern __shared__ float cs[];          // [Dv / 2][2]
   const int t = blockIdx.x, vhalf = Dv >> 1;
   for (int i = threadIdx.x; i < vhalf; i += RP_NT) {
-    const float a = sign * ((float)pos[t] * freqs[i]);
-    cs[2 * i] = cosf(a) * scale;
-    cs[2 * i + 1] = sinf(a) * scale;
+    float sn, c;
+    sincosf(sign * ((float)pos[t] * freqs[i]), &sn, &c);
+    cs[2 * i] = c * scale;
+    cs[2 * i + 1] = sn * scale;
   }
   __syncthreads();
   const AT* row = x + (long)t * H * Dv;

@@ -56,7 +56,7 @@ def test_group_norm_boundary(device, D, groups):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("F", [13, 256, 1000])
+@pytest.mark.parametrize("F", [13, 256, 1000, 8200, 16392])
 def test_polynomial_activation(device, F):
     g = torch.Generator().manual_seed(F)
     z = (torch.randn(6, F, generator=g) * 2).to(torch.bfloat16)
@@ -68,6 +68,8 @@ def test_polynomial_activation(device, F):
         for src in (z.to(device), z.float().to(device), ops.Partial(torch.stack([z.float() * 0.25, z.float() * 0.75]).to(device))):
             out = ops.poly_norm_act(src, c.to(device), 1e-5, out_dtype=torch.float32)
             assert rel(out, want) < 3e-6
+        out16 = ops.poly_norm_act(z.to(device), c.to(device), 1e-5)        # bf16 in and out: the vectorised kernel's shapes
+        assert out16.dtype == torch.bfloat16 and rel(out16, want) < 5e-3
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -80,6 +82,13 @@ def test_sigmoid_gate_reads_columns_of_a_wider_row(device):
         out = ops.sigmoid_mul(xd, wd[:, 21:51], out_dtype=torch.float32)
         want = xd.cpu().to(F64) * oracle.sigmoid(wd.cpu()[:, 21:51].to(F64))
         assert rel(out, want) < 2e-6
+    # 16-bit in and out, widths and offsets in multiples of 8: the vectorised kernel's shapes
+    x8 = torch.randn(5, 64, generator=g).to(torch.bfloat16).to(device)
+    w8 = (torch.randn(5, 200, generator=g) * 4).to(torch.bfloat16).to(device)
+    for c0 in (0, 8, 3):
+        out = ops.sigmoid_mul(x8, w8[:, c0:c0 + 64])
+        want = x8.cpu().to(F64) * oracle.sigmoid(w8.cpu()[:, c0:c0 + 64].to(F64))
+        assert out.dtype == torch.bfloat16 and rel(out, want) < 5e-3
 
 
 @pytest.mark.parametrize("device", DEVICES)
