@@ -296,6 +296,8 @@ class GosuvikModel:
             raise ValueError(f"{p}: a1 / g1 read the layer's input")
         ra, rg = a1.shape[0], g1.shape[0]
         win = torch.cat([sh(p + "q", (Cqk, D)), sh(p + "k", (Cqk, D)), sh(p + "v", (Cv, D)), sh(p + "b", (H, D)), a1, g1], 0)
+        if win.shape[0] % 8:     # rows of zeros up to a multiple of 8: the projection's rows stay 16-byte aligned in bf16
+            win = torch.cat([win, torch.zeros(8 - win.shape[0] % 8, D)], 0)
         L = _Layer(None, self._qw(win), self._qw(sh(p + "o", (D, Cv))))
         L.a2, L.g2 = self._qw(sh(p + "a2", (H * m.dim, ra))), self._qw(sh(p + "g2", (Cv, rg)))
         L.rank_a, L.rank_g = ra, rg

@@ -243,7 +243,8 @@ def cuts_of(T, *sizes):
 @pytest.mark.parametrize("device,dtype", MODES)
 @pytest.mark.parametrize("spec", [dict(heads=4, kv=2, dim=8, vdim=6, conv=3), dict(heads=3, kv=3, dim=5, vdim=7, conv=1),
                                   dict(heads=2, kv=1, dim=64, vdim=64, conv=4), dict(heads=2, kv=2, dim=40, vdim=72, conv=5),
-                                  dict(heads=1, kv=1, dim=200, vdim=16, conv=2)])
+                                  dict(heads=1, kv=1, dim=200, vdim=16, conv=2), dict(heads=8, kv=4, dim=16, vdim=8, conv=4, ra=8, rg=16),
+                                  dict(heads=4, kv=4, dim=128, vdim=128, conv=3, ra=16, rg=8)])
 def test_delta_rule_alone(tmp_path, device, dtype, spec):
     """Whole, in portions down to two rows and one, token by token; the first rows of a sequence (zeros
     before the convolution, zero state), hot rows whose write every later read-out sees."""
@@ -291,7 +292,11 @@ def test_latent_attention_alone(tmp_path, device, dtype, spec):
                                   dict(heads=8, kv=2, dim=64, vdim=64, rot=64, window=17, factor=2.0, scale=0.125, r_heads=4,
                                        r_dim=32, r_vdim=96, cap=10.0),
                                   dict(heads=2, kv=2, dim=32, vdim=16, rot=16, window=0, factor=0, r_heads=1, r_dim=130, r_vdim=20,
-                                       cap=3.0, ls=1.0, rs=1.0)])
+                                       cap=3.0, ls=1.0, rs=1.0),
+                                  dict(heads=4, kv=1, dim=128, vdim=128, rot=64, window=40, scale=0.09, r_heads=2, r_dim=128,
+                                       r_vdim=128),
+                                  dict(heads=6, kv=3, dim=96, vdim=96, rot=96, window=19, scale=0.1, r_heads=1, r_dim=8, r_vdim=8),
+                                  dict(heads=2, kv=2, dim=80, vdim=80, rot=40, window=70, scale=0.11, r_heads=1, r_dim=8, r_vdim=8)])
 def test_parallel_mixer_alone(tmp_path, device, dtype, spec):
     """Sink attention with rotated values beside the matrix memory: hot rows at the window's edge, at
     page borders, far back; portions, decode rows (the split-KV decode kernel where the widths allow)."""
