@@ -421,9 +421,18 @@ static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, i
   // per compute unit (a scan is a chain of dependent steps, so resident waves hide its latencies), up to
   // 32: the sixth butterfly level costs more than the wider launch gains (4 x 2048 rows, 16 heads of
   // 128 x 128: 2.5 ms with 32 lanes, 3.3 ms with 64).
-  const int Cc = Dv >= 64 ? 4 : 1;
+  // Cc: the most columns a thread (a k / q / g value read from LDS then feeds Cc chains) that still leaves
+  // about two waves per SIMD at 16 lanes a group; a prompt batch of few sequences takes 1, a decode batch 4
+  // (4 x 2048 rows, 16 heads of 128 x 128: 2.1 ms with 4 columns a thread, 1.6 with 2, 1.5 with 1).
+  int Cc = 1;
+  if (Dv >= 64)
+    for (int c = 4; c >= 2; c >>= 1)
+      if ((long)nseq * H * Dv / c * 16 / 64 >= 2048) {
+        Cc = c;
+        break;
+      }
   int P = 8;
-  while (P < 64 && (Dk + P - 1) / P > (Cc == 4 ? 8 : 16)) P <<= 1;
+  while (P < 64 && (Dk + P - 1) / P > (Cc >= 2 ? 8 : 16)) P <<= 1;
   if ((Dk + P - 1) / P > 16) return -5;
   while (P < 32 && (Dk + P - 1) / P > 2 && (long)nseq * H * ((Dv + DR_NT / P * Cc - 1) / (DR_NT / P * Cc)) < 1024) P <<= 1;
   const int need = (Dk + P - 1) / P;
@@ -456,6 +465,7 @@ static int delta_launch(const AT* src, long ld, const AT* dec, const AT* gate, i
     else LA_DR_P(16, CC)                                                                                             \
   }
   if (Cc == 4) LA_DR_R(4)
+  else if (Cc == 2) LA_DR_R(2)
   else LA_DR_R(1)
 #undef LA_DR_P
 #undef LA_DR_R

@@ -205,7 +205,7 @@ ORACLE = {"channel_delta": oracle.channel_delta, "latent_attention": oracle.late
 
 def check_mixer(model, layer, W, h, cuts_list, bs, nblocks, dtype, tables=None, must=()):
     """fp32: every row to rounding.  bf16: a row may stand out where 16-bit rounding meets a sharp softmax
-    or a read-out that nearly cancels (one in a hundred), but never a row listed in `must`: the rows
+    or a read-out that nearly cancels (one in fifty), but never a row listed in `must`: the rows
     just inside and just outside a window's edge, where a fault would show."""
     want = ORACLE[layer["type"]](({k: v.to(F64) for k, v in W.items()}), "l0.mix.", layer["mixer"], h.to(F64), 1e-5)
     kv = model.new_kv_cache(nblocks, bs, state_slots=3)
@@ -220,7 +220,7 @@ def check_mixer(model, layer, W, h, cuts_list, bs, nblocks, dtype, tables=None, 
         if dtype == "float32":
             assert float(err.max()) < 1e-4, where
         else:
-            assert int((err > 6e-2).sum()) <= max(1, T // 100) and float(err.median()) < 2e-2, where
+            assert int((err > 6e-2).sum()) <= max(2, T // 50) and float(err.max()) < 2.5 and float(err.median()) < 2e-2, where   # 2: a unit-normed head that changed sign
             for t in must:
                 assert float(err[t]) < 6e-2, (n, t, float(err[t]))
 
@@ -279,11 +279,11 @@ def test_latent_attention_alone(tmp_path, device, dtype, spec):
     a portion and decoded alone, at a page border (pages of 16) and far back (no window)."""
     model, layer, W = build(dense(latent(**spec), 0), 32, tmp_path, device, dtype)
     w = spec["window"] or 1000
-    T = 100
+    T = 100 if spec["window"] else 270          # without a window the hot rows lie hundreds of rows back
     h = inputs(T, 32, 3, hot=(0, 15, 16, 50))
     cuts = [[T], cuts_of(T, 2), [15 + w - 1, 1, 1, 1] + cuts_of(T - 15 - w - 2, 9, 1) if 15 + w + 2 < T else cuts_of(T, 31, 1),
-            [40] + [1] * 60]
-    check_mixer(model, layer, W, h, cuts, 16, 8, dtype, must=edges((0, 15, 16, 50), w, T))
+            [T - 60] + [1] * 60]
+    check_mixer(model, layer, W, h, cuts, 16, T // 16 + 2, dtype, must=edges((0, 15, 16, 50), w, T))
 
 
 @pytest.mark.parametrize("device,dtype", MODES)
