@@ -26,10 +26,6 @@ def rel(got, want):
     return float((got - want).norm() / want.norm().clamp_min(1e-12))
 
 
-def tol(dtype):
-    return 2e-5 if dtype in ("float32", torch.float32) else 2e-2
-
-
 # ------------------------------------------------------------------------------------------- operators
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("D,groups", [(48, 4), (36, 3), (40, 1), (35, 5), (256, 8), (2048, 2), (4100, 4), (96, 96)])
